@@ -8,7 +8,7 @@
 * linked into one shared object next to ``lumen/__init__.py`` so it travels with the repo
   snapshot to the GPU box (no JIT cache under ~/.cache).
 
-Usage: ``python -m lumen.csrc.build [-j N] [--force] [--asm]``.
+Usage: ``python -m lumen.csrc.build [-j N] [--force]``.
 """
 from __future__ import annotations
 
@@ -112,7 +112,7 @@ def _run(cmd):
     return time.time() - t0, r.stderr
 
 
-def build(jobs: int = 8, force: bool = False, asm: bool = False, verbose: bool = True,
+def build(jobs: int = 8, force: bool = False, verbose: bool = True,
           build_dir: str = None, out: str = None) -> str:
     """Compile + link under an exclusive file lock next to the output ``.so``.
 
@@ -132,12 +132,12 @@ def build(jobs: int = 8, force: bool = False, asm: bool = False, verbose: bool =
         if verbose and time.time() - t0 > 1.0:
             print(f"[lumen.build] waited {time.time() - t0:.1f}s for a concurrent build", flush=True)
         try:
-            return _build_locked(jobs, force, asm, verbose, build_dir, out)
+            return _build_locked(jobs, force, verbose, build_dir, out)
         finally:
             fcntl.flock(lk.fileno(), fcntl.LOCK_UN)
 
 
-def _build_locked(jobs, force, asm, verbose, build_dir, out) -> str:
+def _build_locked(jobs, force, verbose, build_dir, out) -> str:
     headers = glob.glob(os.path.join(HERE, "kernels", "*.h"))
     common = ["-O3", "-fPIC", "-std=c++17"]
     jobs_list = []
@@ -148,8 +148,6 @@ def _build_locked(jobs, force, asm, verbose, build_dir, out) -> str:
         if force or _newer([src] + headers, obj):
             cmd = [HIPCC, f"--offload-arch={ARCH}", "-munsafe-fp-atomics", *common, "-c", src,
                    "-o", obj]
-            if asm:
-                cmd.insert(1, "-save-temps")
             jobs_list.append(cmd)
     cpu_src = os.path.join(HERE, "cpu", "cpu_adam.cpp")
     cpu_obj = os.path.join(build_dir, "cpu_adam.o")
@@ -197,9 +195,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("-j", "--jobs", type=int, default=int(os.environ.get("MAX_JOBS", "8")))
     ap.add_argument("--force", action="store_true")
-    ap.add_argument("--asm", action="store_true", help="keep .s (-save-temps) for inspection")
     a = ap.parse_args()
-    build(jobs=a.jobs, force=a.force, asm=a.asm)
+    build(jobs=a.jobs, force=a.force)
 
 
 if __name__ == "__main__":

@@ -685,11 +685,11 @@ __global__ void __launch_bounds__(256) kv_dequant_kernel(
 }
 
 // The PF kernel's inline-asm K / V loads are invisible to hipcc's register allocator, so a spill
-// or copy of a result before its counted wait would read stale data (scripts/tools/
-// check_asm_loads.py audits the code object).  The audit passes for D = 128 (every G) and G = 1
-// (every D); under the register pressure of D = 32 / 64 / 256 with G > 1 hipcc spills the loaded
-// registers right after the issue, so those shapes run the compiler-visible UNI kernel -- and
-// the PF form is not even instantiated for them.
+// or copy of a result before its counted wait would read stale data.  The PF form is therefore
+// kept to the shapes with the least register pressure, D = 128 (every G) and G = 1 (every D);
+// D = 32 / 64 / 256 with G > 1 run the compiler-visible UNI kernel -- the PF form is not even
+// instantiated for them -- and a GPU test compares both forms with the fp32 reference at every
+// head size and group.
 template <int D, int G>
 constexpr bool pa_pf_ok() { return D == 128 || G == 1; }
 

@@ -1501,7 +1501,7 @@ def test_fused_mlp_autograd_matches_unfused(monkeypatch):
 def test_paged_decode_uniform_variants_all_shapes(D, G):
     """The uniform-block-id decode (LUMEN_PA_1PASS 2) and its pipelined inline-asm form (3) at
     the block size that enables them (256 / (D / 8) rows), every head size and GQA group: the
-    pipelined form runs where scripts/tools/check_asm_loads.py passes (D = 128 or G = 1) and
+    pipelined form runs for D = 128 or G = 1 and
     falls back to variant 2 elsewhere -- both must match the fp32 reference at several
     partition sizes."""
     from lumen.ops.attention import paged_decode, paged_decode_ref, write_kv_cache
