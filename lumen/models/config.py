@@ -17,7 +17,7 @@ from typing import Optional
 
 @dataclass
 class ModelConfig:
-    arch: str = "llama"  # "llama" | "opt"
+    arch: str = "llama"  # "llama" | "opt" | "gedatar"
     vocab_size: int = 32000
     hidden_size: int = 4096
     intermediate_size: int = 11008
@@ -37,6 +37,16 @@ class ModelConfig:
     bos_token_id: int = 1
     eos_token_id: int = 2
     name: str = "custom"
+    # Gedatar (hybrid stack: every layer names its own mixer and feed-forward):
+    # layer_specs[i] = {"type": "attention" | "wkv" | "general_delta", "mixer": {...},
+    # "mlp": {...} | None}, exactly as the checkpoint's config.json lists them
+    layer_specs: Optional[list] = None
+    canon_taps: int = 0          # taps of the causal depthwise convolution on the mixer input
+
+    @property
+    def is_hybrid(self) -> bool:
+        """Layers carry per-sequence recurrent state next to (or instead of) a paged K cache."""
+        return self.arch == "gedatar"
 
     @property
     def head_dim(self) -> int:
@@ -53,6 +63,16 @@ class ModelConfig:
     def num_params(self) -> int:
         """Total parameter count (base model, no adapters)."""
         h, v, L = self.hidden_size, self.vocab_size, self.num_hidden_layers
+        if self.arch == "gedatar":
+            from .gedatar import tensor_shapes
+
+            n = 0
+            for shape in tensor_shapes(self).values():
+                k = 1
+                for d in shape:
+                    k *= d
+                n += k
+            return n
         if self.arch == "llama":
             attn = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
             mlp = 3 * h * self.intermediate_size
@@ -79,7 +99,37 @@ class ModelConfig:
         return cls(**{k: v for k, v in d.items() if k in names})
 
 
+def _gedatar_to_config(d: dict) -> ModelConfig:
+    """config.json of a Gedatar checkpoint: {"architecture": "Gedatar", "vocab", "width",
+    "norm": {"eps"}, "canon": {"taps"}, "layers": [{"type", "mixer", "mlp"}, ...]}."""
+    layers = d["layers"]
+    if not layers:
+        raise ValueError("a Gedatar config needs at least one layer")
+    for i, L in enumerate(layers):
+        if L.get("type") not in ("attention", "wkv", "general_delta"):
+            raise ValueError(f"layer {i}: unknown mixer type {L.get('type')!r}")
+        kind = (L.get("mlp") or {}).get("kind", None)
+        if L.get("mlp") is not None and kind not in ("dense", "moe"):
+            raise ValueError(f"layer {i}: unknown feed-forward kind {kind!r}")
+    return ModelConfig(
+        arch="gedatar", vocab_size=int(d["vocab"]), hidden_size=int(d["width"]),
+        num_hidden_layers=len(layers), rms_norm_eps=float(d["norm"]["eps"]),
+        canon_taps=int(d["canon"]["taps"]), layer_specs=layers, intermediate_size=0,
+        num_attention_heads=0, num_key_value_heads=0, max_position_embeddings=1 << 20,
+        bos_token_id=int(d.get("bos_token_id", 0)), eos_token_id=int(d.get("eos_token_id", -1)),
+        pad_token_id=int(d.get("pad_token_id", 0)), name=d.get("_name_or_path", "gedatar"))
+
+
+def gedatar_to_dict(cfg: ModelConfig) -> dict:
+    """The checkpoint form of a Gedatar configuration (inverse of ``_gedatar_to_config``)."""
+    return {"architecture": "Gedatar", "vocab": cfg.vocab_size, "width": cfg.hidden_size,
+            "norm": {"eps": cfg.rms_norm_eps}, "canon": {"taps": cfg.canon_taps},
+            "layers": cfg.layer_specs, "eos_token_id": cfg.eos_token_id}
+
+
 def _hf_to_config(d: dict) -> ModelConfig:
+    if d.get("architecture") == "Gedatar":
+        return _gedatar_to_config(d)
     mt = d.get("model_type", "llama")
     if mt == "opt":
         return ModelConfig(
@@ -153,6 +203,23 @@ PRESETS = {
     "tiny-llama-tp8": dict(arch="llama", vocab_size=1024, hidden_size=512, intermediate_size=2048,
                            num_hidden_layers=2, num_attention_heads=8, num_key_value_heads=8,
                            max_position_embeddings=512, name="tiny-llama-tp8"),
+    # hybrid stack at toy size: chunked sink attention (GQA), RWKV-style and generalized-delta
+    # recurrences, dense and mixture-of-experts feed-forwards, one layer without a feed-forward
+    "tiny-gedatar": dict(
+        arch="gedatar", vocab_size=320, hidden_size=128, num_hidden_layers=4,
+        rms_norm_eps=1e-5, canon_taps=4, intermediate_size=0, num_attention_heads=0,
+        num_key_value_heads=0, max_position_embeddings=1 << 20, eos_token_id=-1,
+        name="tiny-gedatar", layer_specs=[
+            {"type": "wkv", "mixer": {"heads": 2, "dim": 32},
+             "mlp": {"kind": "dense", "ff": 192}},
+            {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 32,
+                                            "scale": 0.2, "mask": {"size": 24}},
+             "mlp": {"kind": "moe", "router": {"experts": 6, "top": 3}, "expert": {"ff": 64},
+                     "shared": {"ff": 96}}},
+            {"type": "general_delta", "mixer": {"heads": 2, "dim": 48}, "mlp": None},
+            {"type": "attention", "mixer": {"heads": 2, "kv_heads": 2, "dim": 64, "vdim": 64,
+                                            "scale": 0.1, "mask": {"size": 40}},
+             "mlp": {"kind": "dense", "ff": 160}}]),
     "tiny-opt": dict(arch="opt", vocab_size=512, hidden_size=64, intermediate_size=256,
                      ffn_dim=256, num_hidden_layers=2, num_attention_heads=4,
                      num_key_value_heads=4, max_position_embeddings=256, word_embed_proj_dim=64,
@@ -180,7 +247,7 @@ def get_config(name_or_path: str) -> ModelConfig:
         cfg_path = os.path.join(name_or_path, "config.json")
         with open(cfg_path) as f:
             d = json.load(f)
-        if "arch" in d and "model_type" not in d:
+        if "arch" in d and "model_type" not in d and "architecture" not in d:
             return ModelConfig.from_dict(d)
         return _hf_to_config(d)
     raise ValueError(f"unknown model '{name_or_path}' (presets: {sorted(PRESETS)})")

@@ -503,3 +503,69 @@ def flash_attention_ref(qkv, cu, nh, nkv, D, causal=True):
         o = F.scaled_dot_product_attention(q, k, v, is_causal=causal)
         outs.append(o[0].transpose(0, 1).reshape(n, nh * D))
     return torch.cat(outs, 0)
+
+
+# ---- keys-as-values attention over a paged key cache, block-diagonal mask, optional sink ------
+# The cache holds ONE tensor per layer, the un-normalised keys [blocks, block_size, G, D]
+# (token-major: a token's keys of all heads are one row), because the values ARE those keys;
+# the unit-RMS key the scores use is recomputed from the row the kernel loads anyway, so the
+# cache costs half the bytes of a K + V cache.  Row i of a sequence sees key j when j <= i and
+# (chunk == 0 or j // chunk == i // chunk); chunks count from position 0 of the sequence.  With
+# ``sink`` the softmax denominator gains exp(0): a key of score 0 that carries no value.
+# (HIP: ``csrc/seqmix/attention.hip``; scores, softmax and the q / k norms in fp32.)
+def write_key_cache(k: torch.Tensor, cache: torch.Tensor, slots: torch.Tensor) -> None:
+    """Rows of k [T, G * D] (any row stride) into cache rows ``slots`` (int64; -1 skips)."""
+    from ._seqmix import DT, call, use_seqmix
+
+    GD = cache.shape[2] * cache.shape[3]
+    if not use_seqmix(k):
+        ok = slots >= 0
+        cache.view(-1, GD)[slots[ok]] = k[ok].to(cache.dtype)
+        return
+    assert k.stride(1) == 1 and cache.is_contiguous() and cache.dtype == k.dtype
+    call("sm_write_k", DT[k.dtype], k, k.stride(0), cache, slots, k.shape[0], GD)
+
+
+def chunk_sink_attention_ref(q, cache, seg, H, G, D, scale, chunk, eps, sink=True):
+    T = q.shape[0]
+    bs = cache.shape[1]
+    out = torch.zeros(T, H, D, dtype=torch.float32, device=q.device)
+    qf = q.float().reshape(T, H, D)
+    qf = qf / torch.sqrt((qf * qf).mean(-1, keepdim=True) + eps)
+    row_seg, pos = seg.row_seg.tolist(), seg.positions.tolist()
+    rows = cache.view(-1, G, D)
+    for t in range(T):
+        i = pos[t]
+        lo = (i // chunk) * chunk if chunk else 0
+        js = torch.arange(lo, i + 1, device=q.device)
+        tbl = seg.tables[row_seg[t]].long()
+        kr = rows[tbl[js // bs] * bs + js % bs].float()            # [n, G, D] raw keys = values
+        kn = kr / torch.sqrt((kr * kr).mean(-1, keepdim=True) + eps)
+        for h in range(H):
+            g = h // (H // G)
+            s = (kn[:, g] @ qf[t, h]) * scale
+            m = torch.clamp(s.max(), min=0.0) if sink else s.max()
+            e = torch.exp(s - m)
+            den = e.sum() + (torch.exp(-m) if sink else 0.0)
+            out[t, h] = (e / den) @ kr[:, g]
+    return out.reshape(T, H * D).to(q.dtype)
+
+
+def chunk_sink_attention(q: torch.Tensor, cache: torch.Tensor, seg, H: int, G: int, D: int,
+                         scale: float, chunk: int, eps: float, sink: bool = True) -> torch.Tensor:
+    """q [T, H * D] (rows may be strided) against the paged raw-key cache; the step's own keys
+    must already be in the cache (``write_key_cache``).  Returns [T, H * D] in q's dtype."""
+    from ._seqmix import DT, call, use_seqmix
+
+    if not use_seqmix(q):
+        return chunk_sink_attention_ref(q, cache, seg, H, G, D, scale, chunk, eps, sink)
+    assert q.stride(1) == 1 and cache.is_contiguous() and cache.dtype == q.dtype
+    assert cache.shape[2] == G and cache.shape[3] == D and H % G == 0
+    if D > 256:
+        raise ValueError(f"attention head size {D} > 256 is not supported")
+    T = q.shape[0]
+    out = torch.empty(T, H * D, dtype=q.dtype, device=q.device)
+    call("sm_chunk_attn", DT[q.dtype], q, q.stride(0), cache, out, seg.tables,
+         seg.tables.shape[1], seg.row_seg, seg.positions, T, H, G, D, cache.shape[1], scale, eps,
+         chunk, int(sink))
+    return out

@@ -80,3 +80,49 @@ def layer_norm(x, w, b, eps):
     """OPT LayerNorm (torch op); frozen params enter autograd as detached aliases."""
     fz = lambda t: t if (t is None or t.requires_grad) else t.detach()  # noqa: E731
     return torch.nn.functional.layer_norm(x, (x.shape[-1],), fz(w), fz(b), eps)
+
+
+# ---- Dynamic Tanh (DyT): tanh(alpha * x) * w + b, no mean or variance ------------------------
+# A DyT norm is the triple (w [W], b [W], alpha [] ) of fp32 tensors; alpha stays on the device
+# (the kernels read it there, so a captured graph never bakes a value in).  Everything is
+# computed in fp32; only the result is rounded to ``out_dtype``.
+def dyt_ref(x, norm, out_dtype=None):
+    w, b, alpha = norm
+    y = torch.tanh(alpha.float() * x.float()) * w.float() + b.float()
+    return y.to(out_dtype or x.dtype)
+
+
+def dyt(x: torch.Tensor, norm, out_dtype=None) -> torch.Tensor:
+    """DyT of the rows of ``x`` [rows, W] (fp32 or 16-bit) in ``out_dtype``."""
+    from ._seqmix import DT, call, use_seqmix
+
+    out_dtype = out_dtype or x.dtype
+    if not use_seqmix(x):
+        return dyt_ref(x, norm, out_dtype)
+    x = x.contiguous()
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    call("sm_dyt", DT[x.dtype], DT[out_dtype], x, norm[0], norm[1], norm[2], out,
+         x.numel() // x.shape[-1], x.shape[-1])
+    return out
+
+
+def dyt_residual_ref(x, y, post, pre=None, out_dtype=None):
+    x.add_(dyt_ref(y, post, torch.float32))
+    return x, (dyt_ref(x, pre, out_dtype or y.dtype) if pre is not None else None)
+
+
+def dyt_residual(x: torch.Tensor, y: torch.Tensor, post, pre=None, out_dtype=None):
+    """The fp32 residual stream ``x`` [T, W] takes a sublayer's output in place,
+    x += DyT_post(y), and -- fused -- the next sublayer's input h = DyT_pre(x) is produced in
+    ``out_dtype``.  Returns (x, h or None)."""
+    from ._seqmix import DT, call, use_seqmix
+
+    out_dtype = out_dtype or y.dtype
+    if not use_seqmix(x):
+        return dyt_residual_ref(x, y, post, pre, out_dtype)
+    assert x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous()
+    h = torch.empty(x.shape, dtype=out_dtype, device=x.device) if pre is not None else None
+    p = pre or (None, None, None)
+    call("sm_dyt_residual", DT[y.dtype], DT[out_dtype], x, y, post[0], post[1], post[2], h,
+         p[0], p[1], p[2], x.shape[0], x.shape[1])
+    return x, h

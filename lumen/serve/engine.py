@@ -158,7 +158,14 @@ class LLMEngine:
             from ..parallel.dist import host_group
 
             host_group()
-        self.weights = ServeWeights(model, self.rank, self.tp)
+        self.hybrid = bool(getattr(model.config, "is_hybrid", False))
+        if self.hybrid:
+            self._check_hybrid_options()
+            from .hybrid_runner import HybridWeights
+
+            self.weights = HybridWeights(model, self.rank, self.tp)
+        else:
+            self.weights = ServeWeights(model, self.rank, self.tp)
         if cfg.kv_cache_dtype not in ("auto", "fp8"):
             raise ValueError(f"kv_cache_dtype must be 'auto' or 'fp8', got {cfg.kv_cache_dtype}")
         self.kv_dtype = torch.float8_e4m3fn if cfg.kv_cache_dtype == "fp8" else dt
@@ -184,10 +191,20 @@ class LLMEngine:
             car = maybe_custom_allreduce(
                 tp_group, dev, max(8 << 20, rows * model.config.hidden_size * esz,
                                    rows * vshard * esz))
-        self.runner = ModelRunner(self.weights, nb, cfg.block_size, dev, cfg.max_model_len,
-                                  tp_group, use_graphs=cfg.use_graphs,
-                                  max_graph_batch=min(256, cfg.max_num_seqs), custom_ar=car,
-                                  kv_dtype=self.kv_dtype)
+        self.states = None
+        if self.hybrid:
+            from .hybrid_runner import HybridRunner
+            from .state_manager import StateSlots
+
+            self.states = StateSlots(cfg.max_num_seqs)
+            self.runner = HybridRunner(self.weights, nb, cfg.block_size, dev, cfg.max_model_len,
+                                       state_slots=cfg.max_num_seqs, use_graphs=cfg.use_graphs,
+                                       max_graph_batch=min(256, cfg.max_num_seqs))
+        else:
+            self.runner = ModelRunner(self.weights, nb, cfg.block_size, dev, cfg.max_model_len,
+                                      tp_group, use_graphs=cfg.use_graphs,
+                                      max_graph_batch=min(256, cfg.max_num_seqs), custom_ar=car,
+                                      kv_dtype=self.kv_dtype)
         self.lora_names: List[str] = []
         if cfg.lora_modules:
             from .multi_lora import MultiLoRA
@@ -208,7 +225,7 @@ class LLMEngine:
         self.scheduler = Scheduler(SchedulerConfig(
             cfg.max_num_seqs, cfg.max_num_batched_tokens, cfg.max_model_len,
             prefill_boost=max(1, int(cfg.prefill_boost)), policy=cfg.scheduling_policy),
-            self.blocks)
+            self.blocks, self.states)
         if tokenizer is None:
             from ..data.tokenizer import load_tokenizer
 
@@ -221,9 +238,29 @@ class LLMEngine:
                       "spec_accepted": 0, "spec_steps": 0}
 
     # --------------------------------------------------------------------------------------
+    def _check_hybrid_options(self) -> None:
+        """Options that assume every layer's state is a per-token cache: refused for a hybrid
+        model, whose recurrent state cannot be shared by prefix or rolled back after a rejected
+        draft."""
+        c = self.cfg
+        bad = [n for n, on in (("tp_size > 1", c.tp_size > 1),
+                               ("enable_prefix_caching", c.enable_prefix_caching),
+                               ("num_speculative_tokens", c.num_speculative_tokens > 0),
+                               ("lora_modules", bool(c.lora_modules)),
+                               ("adapter", bool(c.adapter)),
+                               ("kv_cache_dtype fp8", c.kv_cache_dtype == "fp8")) if on]
+        if bad:
+            raise ValueError(f"not supported for hybrid (recurrent-state) models: {', '.join(bad)}")
+
     def _auto_blocks(self, dt) -> int:
-        per_tok = kv_bytes_per_token(self.model_config, torch.tensor([], dtype=dt).element_size(),
-                                     self.tp)
+        if self.hybrid:
+            from .hybrid_runner import key_bytes_per_token
+
+            per_tok = key_bytes_per_token(self.model_config,
+                                          torch.tensor([], dtype=dt).element_size())
+        else:
+            per_tok = kv_bytes_per_token(self.model_config,
+                                         torch.tensor([], dtype=dt).element_size(), self.tp)
         per_block = per_tok * self.cfg.block_size
         if self.device.type == "cuda":
             free, total = torch.cuda.mem_get_info(self.device)
@@ -376,6 +413,26 @@ class LLMEngine:
             extra.append(np.asarray(prows, dtype=np.int64))
         if use_lora:
             extra.append(np.concatenate(lora))
+        seg_n = 0
+        if self.hybrid:
+            # segments of the step (ops.segments.SegBatch): one per prefill chunk, one per decode
+            # row -- row offsets, state slot, first position, row -> segment, block tables
+            S = P + N
+            lens_s = np.asarray([c for _, c in batch.prefills] + [1] * N, dtype=np.int64)
+            seg_cu = np.concatenate([[0], np.cumsum(lens_s)])
+            seg_slot = np.fromiter((self.states.slot(s.seq_id) for s in batch.seqs), np.int64, S)
+            seg_start = np.asarray([s.num_cached for s, _ in batch.prefills]
+                                   + [s.length - 1 for s in batch.decodes], dtype=np.int64)
+            maxb = max(maxb_p, maxb_d)
+            seg_tbl = np.zeros((S, maxb), dtype=np.int64)
+            for i, t in enumerate(ptables):
+                seg_tbl[i, :len(t)] = t
+            if N:
+                seg_tbl[P:, :maxb_d] = dec_bt
+            seg_arrays = [seg_cu, seg_slot, seg_start, np.repeat(np.arange(S), lens_s),
+                          seg_tbl.reshape(-1)]
+            seg_n = sum(a.size for a in seg_arrays)
+            extra += seg_arrays
         host = np.concatenate([np.concatenate(parts)] + extra)
         dev = self._to_device(host)
         o = 3 * T
@@ -413,6 +470,14 @@ class LLMEngine:
             o += len(prows)
         if use_lora:
             inp.lora_ids = dev[o:o + T].int()
+            o += T
+        if self.hybrid:
+            from ..ops.segments import SegBatch
+
+            g = dev[o:o + seg_n].int()
+            inp.seg = SegBatch(g[:S + 1], g[S + 1:2 * S + 1], g[2 * S + 1:3 * S + 1],
+                               g[3 * S + 1:3 * S + 1 + T], inp.positions,
+                               g[3 * S + 1 + T:].view(S, maxb), inp.slots)
         return inp
 
     def _to_device(self, host: "np.ndarray") -> torch.Tensor:

@@ -1,0 +1,295 @@
+"""Serving runner for hybrid stacks (Gedatar): paged key cache + per-sequence recurrent state.
+
+One step function for prefill chunks, decode rows and mixtures of both.  The rows of a step are
+cut into segments (``ops.segments.SegBatch``: one per chunk, one per decode row); per layer
+
+    h  = DyT + causal depthwise conv (HIP, one pass; conv tails per state slot)
+    y  = mixer(h):  attention      q|k GEMM -> keys into the paged cache -> chunk/sink attention
+                    wkv            token shift -> r,k,v,g GEMMs + decay GEMMs -> scan (HIP)
+                    general_delta  one fused r|k|v|g|a|w1 GEMM + decay GEMM -> scan (HIP)
+         -> output GEMM
+    x += DyT(y); h2 = DyT(x)           (HIP, fused)
+    y2 = feed-forward(h2): gate|up GEMM -> gated activation (x routing weight) -> down GEMM
+    x += DyT(y2)
+The residual stream x, every norm, the router, the scores and the recurrences are fp32; GEMMs and
+their activations run in the model dtype (bf16 with fp32 accumulation, or true fp32).
+
+State (``HybridState``) is indexed by the slot ``serve.state_manager.StateSlots`` gives a sequence
+while it runs: conv tails [slots, taps - 1, W] for every layer, the previous row [slots, W] and
+the matrix state [slots, H, D, D] of the recurrent mixers.  Nothing is cleared when a slot is
+handed to a new sequence: a segment that starts at position 0 reads zeros instead of the slot.
+Attention layers keep un-normalised keys only (the values are the keys) in a cache paged by the
+engine's BlockManager, [blocks, block_size, kv_heads, dim] per layer.
+
+Pure decode steps replay a hipGraph per batch bucket (ModelRunner.decode), the segment tensors
+being static buffers; padding rows use the spare state slot and write no keys.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
+
+import torch
+import torch.nn.functional as F
+
+from ..models.config import ModelConfig
+from ..models.gedatar import DELTA_DECAY, DELTA_KEY_EPS
+from ..ops.attention import chunk_sink_attention, write_key_cache
+from ..ops.conv import dyt_canon
+from ..ops.moe import gated_act, route_topk
+from ..ops.norm import dyt, dyt_residual
+from ..ops.recurrent import delta_scan, token_shift, wkv_scan
+from ..ops.segments import SegBatch, whole_sequences
+from .model_runner import ModelRunner, StepInput
+
+
+@dataclass
+class HybridLayerW:
+    kind: str                       # attention | wkv | general_delta
+    m: dict                         # the mixer's sizes and constants
+    norms: Dict[str, tuple]         # norm1 / norm1b / norm2 / norm2b -> (w, b, alpha) fp32
+    canon: torch.Tensor             # [W, taps] fp32
+    w: Dict[str, torch.Tensor] = field(default_factory=dict)
+    ff: Optional[dict] = None       # feed-forward: E, top, ff, ffs, gu, down, router, router_b
+
+
+class HybridWeights:
+    """Inference weights of a GedatarForCausalLM: projections that share an input are stacked
+    into one GEMM; norm weights, biases, decay offsets and the router are kept in fp32."""
+
+    def __init__(self, model, tp_rank: int = 0, tp_size: int = 1):
+        if tp_size != 1:
+            raise NotImplementedError("hybrid models are served at tensor-parallel size 1")
+        cfg: ModelConfig = model.config
+        self.cfg = cfg
+        t = model.tensor
+        f32 = lambda n: t(n).detach().float().contiguous()  # noqa: E731
+        norm = lambda n: (f32(n), f32(n + ".b"), f32(n + ".alpha"))  # noqa: E731
+        self.dtype = t("embed").dtype
+        self.embed = t("embed").detach()
+        self.final = norm("final.norm")
+        self.lm_head = t("head").detach()
+        self.vocab_shard = cfg.vocab_size
+        self.layers: List[HybridLayerW] = []
+        with torch.no_grad():
+            for i, spec in enumerate(cfg.layer_specs):
+                p = f"l{i}."
+                x = p + "mix."
+                m = spec["mixer"]
+                names = ("norm1", "norm1b") + (("norm2", "norm2b") if spec.get("mlp") else ())
+                L = HybridLayerW(spec["type"], m, {n: norm(p + n) for n in names},
+                                 f32(p + "canon1"))
+                if L.kind == "attention":
+                    L.w["qk"] = torch.cat([t(x + "q"), t(x + "k")], 0).contiguous()
+                elif L.kind == "wkv":
+                    L.w["mu"] = torch.stack([f32(x + "mu." + s) for s in "rkvgw"]).contiguous()
+                    L.w["rkvg"] = torch.stack([t(x + s).t() for s in "rkvg"]).contiguous()
+                    L.w["w1"], L.w["w2"] = t(x + "w1").detach(), t(x + "w2").detach()
+                    L.w["u"] = f32(x + "u")
+                else:
+                    L.w["in"] = torch.cat([t(x + s) for s in ("r", "k", "v", "g", "a", "w1")],
+                                          0).contiguous()
+                    L.w["w2"] = t(x + "w2").detach()
+                    L.w["a_b"] = f32(x + "a.b")
+                if L.kind != "attention":
+                    L.w["w0"], L.w["norm"] = f32(x + "w0"), f32(x + "norm")
+                L.w["o"] = t(x + "o").detach()
+                f = spec.get("mlp")
+                if f:
+                    y = p + "mlp."
+                    if f["kind"] == "dense":
+                        L.ff = dict(E=0, top=0, ff=0, ffs=f["ff"],
+                                    gu=torch.cat([t(y + "gate"), t(y + "up")], 0).contiguous(),
+                                    down=t(y + "down").detach())
+                    else:
+                        E, top = f["router"]["experts"], f["router"]["top"]
+                        ffe = f["expert"]["ff"]
+                        ffs = f["shared"]["ff"] if f.get("shared") else 0
+                        gu = [w for e in range(E) for w in (t(y + f"e{e}.gate"), t(y + f"e{e}.up"))]
+                        dn = [t(y + f"e{e}.down") for e in range(E)]
+                        if ffs:
+                            gu += [t(y + "shared.gate"), t(y + "shared.up")]
+                            dn.append(t(y + "shared.down"))
+                        L.ff = dict(E=E, top=top, ff=ffe, ffs=ffs, gu=torch.cat(gu, 0).contiguous(),
+                                    down=torch.cat(dn, 1).contiguous(), router=f32(y + "router"),
+                                    router_b=f32(y + "router.b"))
+                self.layers.append(L)
+
+
+class HybridState:
+    """Per-layer caches of a hybrid model: ``slots`` sequences of recurrent state (+ one spare
+    slot for graph padding rows) and ``num_blocks`` pages of keys for the attention layers."""
+
+    def __init__(self, w: HybridWeights, slots: int, num_blocks: int, block_size: int, device):
+        cfg = w.cfg
+        W, K = cfg.hidden_size, max(cfg.canon_taps - 1, 0)
+        f32 = dict(dtype=torch.float32, device=device)
+        self.slots = slots
+        self.spare = slots
+        self.tail = [torch.zeros(slots + 1, K, W, **f32) for _ in w.layers]
+        self.prev: List[Optional[torch.Tensor]] = []
+        self.S: List[Optional[torch.Tensor]] = []
+        self.keys: List[Optional[torch.Tensor]] = []
+        for L in w.layers:
+            m = L.m
+            rec = L.kind != "attention"
+            self.prev.append(torch.zeros(slots + 1, W, **f32) if L.kind == "wkv" else None)
+            self.S.append(torch.zeros(slots + 1, m["heads"], m["dim"], m["dim"], **f32)
+                          if rec else None)
+            self.keys.append(None if rec else torch.zeros(
+                num_blocks, block_size, m["kv_heads"], m["dim"], dtype=w.dtype, device=device))
+
+
+def key_bytes_per_token(cfg: ModelConfig, dtype_bytes: int = 2) -> int:
+    return max(1, sum(L["mixer"]["kv_heads"] * L["mixer"]["dim"] for L in cfg.layer_specs
+                      if L["type"] == "attention") * dtype_bytes)
+
+
+def state_bytes_per_slot(cfg: ModelConfig) -> int:
+    n = 0
+    for L in cfg.layer_specs:
+        n += max(cfg.canon_taps - 1, 0) * cfg.hidden_size
+        if L["type"] != "attention":
+            n += L["mixer"]["heads"] * L["mixer"]["dim"] ** 2
+        if L["type"] == "wkv":
+            n += cfg.hidden_size
+    return 4 * n
+
+
+def run_layers(w: HybridWeights, st: HybridState, tokens: torch.Tensor, seg: SegBatch,
+               observe=None) -> torch.Tensor:
+    """The step function: token ids [T] + their segments -> the fp32 residual stream [T, W]
+    after the last layer.  State and key cache in ``st`` move on by the step's rows."""
+    cfg = w.cfg
+    dt = w.dtype
+    eps = cfg.rms_norm_eps
+    x = F.embedding(tokens, w.embed).float()
+    for i, L in enumerate(w.layers):
+        m = L.m
+        h = dyt_canon(x, L.norms["norm1"], L.canon, st.tail[i], seg, dt)
+        if L.kind == "attention":
+            H, G, D = m["heads"], m["kv_heads"], m["dim"]
+            qk = F.linear(h, L.w["qk"])
+            write_key_cache(qk[:, H * D:], st.keys[i], seg.cache_slots)
+            o = chunk_sink_attention(qk[:, :H * D], st.keys[i], seg, H, G, D, float(m["scale"]),
+                                     int(m["mask"]["size"]), eps, sink=True)
+        elif L.kind == "wkv":
+            H, D = m["heads"], m["dim"]
+            mix = token_shift(h, L.w["mu"], st.prev[i], seg)
+            rkvg = torch.bmm(mix[:4], L.w["rkvg"])
+            wl = F.linear(torch.tanh(F.linear(mix[4], L.w["w1"])), L.w["w2"])
+            o = wkv_scan(rkvg[0], rkvg[1], rkvg[2], wl, rkvg[3], L.w["w0"], L.w["u"], L.w["norm"],
+                         st.S[i], seg, H, D, eps)
+        else:
+            H, D = m["heads"], m["dim"]
+            HD = H * D
+            z = F.linear(h, L.w["in"])
+            wl = F.linear(torch.tanh(z[:, 5 * HD:]), L.w["w2"])
+            o = delta_scan(z[:, :HD], z[:, HD:2 * HD], z[:, 2 * HD:3 * HD], wl,
+                           z[:, 4 * HD:5 * HD], z[:, 3 * HD:4 * HD], L.w["w0"], L.w["a_b"],
+                           L.w["norm"], st.S[i], seg, H, D, eps, DELTA_DECAY, DELTA_KEY_EPS)
+        y = F.linear(o, L.w["o"])
+        f = L.ff
+        if f is None:
+            x, _ = dyt_residual(x, y, L.norms["norm1b"], None, dt)
+        else:
+            x, h2 = dyt_residual(x, y, L.norms["norm1b"], L.norms["norm2"], dt)
+            wts = None
+            if f["E"]:
+                # the router in fp32, on the (possibly 16-bit rounded) normed row
+                z = torch.addmm(f["router_b"], h2.float(), f["router"].t())
+                wts = route_topk(z, f["top"])
+            act = gated_act(F.linear(h2, f["gu"]), wts, f["E"], f["ff"], f["ffs"])
+            x, _ = dyt_residual(x, F.linear(act, f["down"]), L.norms["norm2b"], None, dt)
+        if observe is not None:
+            observe(i, x)
+    return x
+
+
+class HybridRunner(ModelRunner):
+    """ModelRunner for hybrid stacks: the same step interface (execute / decode / sample, the
+    hipGraph decode buckets), its own weights, caches and step function."""
+
+    def __init__(self, weights: HybridWeights, num_blocks: int, block_size: int,
+                 device: torch.device, max_model_len: int = 4096, state_slots: int = 256,
+                 use_graphs: bool = True, max_graph_batch: int = 256):
+        self.w = weights
+        self.cfg = weights.cfg
+        self.device = device
+        self.block_size = block_size
+        self.num_blocks = num_blocks
+        self.max_model_len = max_model_len
+        self.tp_group, self.tp, self.car, self.lora = None, 1, None, None
+        self.max_blocks = (max_model_len + block_size - 1) // block_size
+        self.kv_dtype = weights.dtype
+        self.state = HybridState(weights, state_slots, num_blocks, block_size, device)
+        self.use_graphs = use_graphs and device.type == "cuda"
+        self.graph_buckets = [b for b in (1, 2, 4, 8, 16, 32, 64, 96, 128, 160, 192, 224, 256)
+                              if b <= max(1, max_graph_batch)]
+        self._graph_gathers = True
+        self._graphs: Dict[int, tuple] = {}
+        self._graph_pool = None
+        self.observe = None   # callable(layer, x) after every layer (debugging / layer dumps)
+
+    def _logits_rows(self, x: torch.Tensor, rows: Optional[torch.Tensor]) -> torch.Tensor:
+        if rows is not None:
+            if rows.numel() == 0:
+                return torch.empty(0, self.cfg.vocab_size, device=x.device, dtype=self.w.dtype)
+            x = x[rows]
+        return F.linear(dyt(x, self.w.final, self.w.dtype), self.w.lm_head)
+
+    @torch.no_grad()
+    def execute(self, inp: StepInput) -> torch.Tensor:
+        x = run_layers(self.w, self.state, inp.tokens, inp.seg, self.observe)
+        if inp.extra_rows is not None and inp.extra_rows.numel():
+            self.extra_logits = self._logits_rows(x, inp.extra_rows)
+        return self._logits_rows(x, inp.sample_rows)
+
+    prefill = execute
+
+    # ---- decode: one row per sequence (graph hooks of ModelRunner.decode) --------------------
+    def _decode_input(self, inp: StepInput) -> torch.Tensor:
+        return self._logits_rows(run_layers(self.w, self.state, inp.tokens, inp.seg,
+                                            self.observe), None)
+
+    def _static_inputs(self, bucket: int) -> dict:
+        dev = self.device
+        i32 = dict(dtype=torch.int32, device=dev)
+        ar = torch.arange(bucket + 1, **i32)
+        return {"tokens": torch.zeros(bucket, dtype=torch.long, device=dev),
+                "seg": SegBatch(ar, torch.full((bucket,), self.state.spare, **i32),
+                                torch.zeros(bucket, **i32), ar[:bucket].clone(),
+                                torch.zeros(bucket, **i32),
+                                torch.zeros(bucket, self.max_blocks, **i32),
+                                torch.full((bucket,), -1, dtype=torch.long, device=dev))}
+
+    def _fill_static(self, st: dict, inp: StepInput, N: int, bucket: int) -> None:
+        sg, src = st["seg"], inp.seg
+        st["tokens"][:N].copy_(inp.tokens)
+        sg.slot[:N].copy_(src.slot)
+        sg.start[:N].copy_(src.start)
+        sg.positions[:N].copy_(src.positions)
+        sg.tables[:N, :src.tables.shape[1]].copy_(src.tables)
+        sg.cache_slots[:N].copy_(src.cache_slots)
+        if N < bucket:  # padding rows: position 0 of the spare state slot, no key written
+            sg.slot[N:].fill_(self.state.spare)
+            sg.start[N:].zero_()
+            sg.positions[N:].zero_()
+            sg.cache_slots[N:].fill_(-1)
+
+    def _decode_static(self, st: dict) -> torch.Tensor:
+        return self._logits_rows(run_layers(self.w, self.state, st["tokens"], st["seg"]), None)
+
+
+@torch.no_grad()
+def forward_fresh(model, input_ids: torch.Tensor, block_size: int = 16) -> torch.Tensor:
+    """Logits [B, S, V] of whole sequences on a private, fresh cache (GedatarForCausalLM.forward)."""
+    B, S = input_ids.shape
+    dev = input_ids.device
+    w = HybridWeights(model)
+    nb = B * ((S + block_size - 1) // block_size)
+    st = HybridState(w, B, nb, block_size, dev)
+    seg = whole_sequences([S] * B, dev, block_size=block_size)
+    x = run_layers(w, st, input_ids.reshape(-1), seg)
+    y = F.linear(dyt(x, w.final, w.dtype), w.lm_head)
+    return y.view(B, S, -1)

@@ -118,6 +118,7 @@ class StepInput:
     top_ks: Optional[torch.Tensor] = None        # [R] int32
     extra_rows: Optional[torch.Tensor] = None    # prompt-logprob rows (TP = 1), int64 [E]
     prompt_meta: Optional[list] = None           # host: (seq, first scored token, count, row)
+    seg: Optional[object] = None                 # ops.segments.SegBatch (hybrid models)
 
     @property
     def num_prefill_rows(self) -> int:
@@ -385,13 +386,38 @@ class ModelRunner:
     def decode(self, inp: StepInput) -> torch.Tensor:
         N = inp.tokens.shape[0]
         if not self.use_graphs or N > self.graph_buckets[-1]:
-            return self._decode_eager(inp.tokens, inp.positions, inp.slots, inp.block_tables,
-                                      inp.context_lens, inp.max_context, inp.lora_ids)
+            return self._decode_input(inp)
         bucket = next(b for b in self.graph_buckets if b >= N)
         g = self._graphs.get(bucket)
         if g is None:
             g = self._capture(bucket)
         graph, st, out = g
+        self._fill_static(st, inp, N, bucket)
+        graph.replay()
+        if self._graph_gathers:
+            return out[:N]
+        # the vocab-parallel gather stays outside the graph when it would need RCCL
+        return self._vocab_gather(out[:N])
+
+    # The three hooks a runner with other per-step inputs (recurrent state slots) overrides:
+    # the eager decode of a StepInput, the static buffers of a captured bucket, and the eager
+    # decode from those buffers (what the graph captures).
+    def _decode_input(self, inp: StepInput) -> torch.Tensor:
+        return self._decode_eager(inp.tokens, inp.positions, inp.slots, inp.block_tables,
+                                  inp.context_lens, inp.max_context, inp.lora_ids)
+
+    def _static_inputs(self, bucket: int) -> dict:
+        dev = self.device
+        st = {"tokens": torch.zeros(bucket, dtype=torch.long, device=dev),
+              "positions": torch.zeros(bucket, dtype=torch.int32, device=dev),
+              "slots": torch.full((bucket,), -1, dtype=torch.long, device=dev),
+              "block_tables": torch.zeros(bucket, self.max_blocks, dtype=torch.int32, device=dev),
+              "context_lens": torch.ones(bucket, dtype=torch.int32, device=dev)}
+        if self.lora is not None:
+            st["lora_ids"] = torch.zeros(bucket, dtype=torch.int32, device=dev)
+        return st
+
+    def _fill_static(self, st: dict, inp: StepInput, N: int, bucket: int) -> None:
         st["tokens"][:N].copy_(inp.tokens)
         st["positions"][:N].copy_(inp.positions)
         st["slots"][:N].copy_(inp.slots)
@@ -403,23 +429,14 @@ class ModelRunner:
         if N < bucket:  # padding rows: no cache write, one-token context on block 0
             st["slots"][N:].fill_(-1)
             st["context_lens"][N:].fill_(1)
-        graph.replay()
-        if self._graph_gathers:
-            return out[:N]
-        # the vocab-parallel gather stays outside the graph when it would need RCCL
-        return self._vocab_gather(out[:N])
+
+    def _decode_static(self, st: dict) -> torch.Tensor:
+        return self._decode_eager(st["tokens"], st["positions"], st["slots"], st["block_tables"],
+                                  st["context_lens"], self.max_model_len, st.get("lora_ids"),
+                                  self._graph_gathers)
 
     def _capture(self, bucket: int):
-        dev = self.device
-        st = {"tokens": torch.zeros(bucket, dtype=torch.long, device=dev),
-              "positions": torch.zeros(bucket, dtype=torch.int32, device=dev),
-              "slots": torch.full((bucket,), -1, dtype=torch.long, device=dev),
-              "block_tables": torch.zeros(bucket, self.max_blocks, dtype=torch.int32, device=dev),
-              "context_lens": torch.ones(bucket, dtype=torch.int32, device=dev)}
-        if self.lora is not None:
-            st["lora_ids"] = torch.zeros(bucket, dtype=torch.int32, device=dev)
-        args = (st["tokens"], st["positions"], st["slots"], st["block_tables"],
-                st["context_lens"], self.max_model_len, st.get("lora_ids"), self._graph_gathers)
+        st = self._static_inputs(bucket)
         # one warm-up stream for every bucket (per-stream decode-GEMM workspaces stay few)
         s = getattr(self, "_warm_stream", None)
         if s is None:
@@ -427,13 +444,13 @@ class ModelRunner:
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
             for _ in range(2):  # warm up (allocator, hipBLASLt heuristics) outside capture
-                self._decode_eager(*args)
+                self._decode_static(st)
         torch.cuda.current_stream().wait_stream(s)
         graph = torch.cuda.CUDAGraph()
         if self._graph_pool is None:
             self._graph_pool = torch.cuda.graph_pool_handle()
         with torch.cuda.graph(graph, pool=self._graph_pool):
-            out = self._decode_eager(*args)
+            out = self._decode_static(st)
         self._graphs[bucket] = (graph, st, out)
         return self._graphs[bucket]
 

@@ -82,11 +82,14 @@ class Batch:
 class Scheduler:
     POLICIES = ("chunked", "prefill_first")
 
-    def __init__(self, cfg: SchedulerConfig, blocks: BlockManager):
+    def __init__(self, cfg: SchedulerConfig, blocks: BlockManager, states=None):
         if cfg.policy not in self.POLICIES:
             raise ValueError(f"scheduling policy must be one of {self.POLICIES}, got {cfg.policy!r}")
         self.cfg = cfg
         self.blocks = blocks
+        # state_manager.StateSlots of a hybrid model (None otherwise): a sequence holds one
+        # recurrent-state slot exactly as long as it holds cache blocks
+        self.states = states
         self.waiting: Deque[Sequence] = deque()
         self.running: List[Sequence] = []
         self.num_preemptions = 0
@@ -104,6 +107,8 @@ class Scheduler:
                     q.remove(s)
                     s.status, s.finish_reason = Status.FINISHED, "abort"
                     self.blocks.free_seq(s.seq_id)
+                    if self.states is not None:
+                        self.states.release(s.seq_id)
 
     @property
     def has_work(self) -> bool:
@@ -126,6 +131,8 @@ class Scheduler:
             s = self.waiting[0]
             if not self.blocks.can_allocate(s.length + 1):
                 break
+            if self.states is not None and not self.states.num_free:
+                break
             if whole and batch.prefills and not self._fits(s, budget):
                 break   # vLLM 0.6 (no chunked prefill): whole prompts only, FCFS
             d0 = self._first_block(s) if share else None
@@ -140,6 +147,8 @@ class Scheduler:
             s.num_cached = self.blocks.allocate(
                 s.seq_id, s.length + 1,
                 s.all_ids if s.params.prompt_logprobs is None else None, s.lora_slot)
+            if self.states is not None:
+                self.states.alloc(s.seq_id)
             s.prefilled = False
             s.status = Status.RUNNING
             self.running.append(s)
@@ -227,6 +236,8 @@ class Scheduler:
         whose K/V launched steps wrote stay cached (a recomputed or follow-up prompt hits them)."""
         self.blocks.free_seq(s.seq_id, s.all_ids, min(s.num_cached, len(s.all_ids)),
                              s.lora_slot)
+        if self.states is not None:
+            self.states.release(s.seq_id)
 
     def _preempt(self, s: Sequence) -> None:
         self.running.remove(s)
