@@ -191,12 +191,95 @@ def _build_locked(jobs, force, verbose, build_dir, out) -> str:
     return out
 
 
+# ---- the sequence-mixing kernel library (hybrid models) -----------------------------------------
+# ``seqmix/*.hip`` -> ``lumen/_C_seqmix.so``: extern "C" launchers only (bound with ctypes in
+# lumen/ops/_seqmix.py), so it needs neither the torch headers nor the rest of the extension and a
+# first use on a fresh checkout compiles just these files.
+SEQMIX_FLAGS = ["-O3", "-fPIC", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+                "-packed-fp32-ops"]
+
+
+def seqmix_path() -> str:
+    return os.path.join(PKG, "_C_seqmix.so")
+
+
+def seqmix_sources() -> list:
+    d = os.path.join(HERE, "seqmix")
+    return sorted(glob.glob(os.path.join(d, "*.hip")) + glob.glob(os.path.join(d, "*.h"))
+                  + [os.path.join(HERE, "kernels", "common.h")])
+
+
+def seqmix_digest() -> str:
+    import hashlib
+
+    h = hashlib.sha256()
+    for f in seqmix_sources():
+        with open(f, "rb") as fh:
+            h.update(os.path.relpath(f, PKG).encode() + b":" + fh.read())
+    return h.hexdigest()
+
+
+def _seqmix_manifest() -> str:
+    return os.path.join(PKG, "_C_seqmix.sources.json")
+
+
+def seqmix_stale() -> bool:
+    """True when the library is missing or was built from other sources than the tree holds."""
+    import json
+
+    try:
+        with open(_seqmix_manifest()) as f:
+            return json.load(f).get("sha256") != seqmix_digest() or not os.path.exists(seqmix_path())
+    except (OSError, ValueError):
+        return True
+
+
+def build_seqmix(jobs: int = 8, force: bool = False, verbose: bool = True) -> str:
+    """Compile + link ``lumen/_C_seqmix.so`` under the same file-lock / atomic-rename discipline
+    as ``build`` (several processes may need it at once)."""
+    import fcntl
+    import json
+
+    out = seqmix_path()
+    build_dir = os.path.join(os.environ.get("LUMEN_BUILD_DIR") or BUILD, "seqmix")
+    os.makedirs(build_dir, exist_ok=True)
+    with open(out + ".lock", "a+") as lk:
+        fcntl.flock(lk.fileno(), fcntl.LOCK_EX)
+        try:
+            if not force and not seqmix_stale():
+                return out
+            hips = [f for f in seqmix_sources() if f.endswith(".hip")]
+            objs = [os.path.join(build_dir, os.path.basename(f) + ".o") for f in hips]
+            cmds = [[HIPCC, f"--offload-arch={ARCH}", *SEQMIX_FLAGS, "-c", f, "-o", o]
+                    for f, o in zip(hips, objs)]
+            with ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
+                for cmd, (dt, _) in zip(cmds, ex.map(_run, cmds)):
+                    if verbose:
+                        print(f"[lumen.build] seqmix/{os.path.basename(cmd[-3])} {dt:.1f}s",
+                              flush=True)
+            _run([HIPCC, "-shared", "-fPIC", *objs, "-o", out])
+            tmp = _seqmix_manifest() + f".part{os.getpid()}"
+            with open(tmp, "w") as f:
+                json.dump({"sha256": seqmix_digest(), "arch": ARCH,
+                           "built_at": time.strftime("%Y-%m-%dT%H:%M:%S")}, f, indent=1)
+            os.replace(tmp, _seqmix_manifest())
+            if verbose:
+                print(f"[lumen.build] linked {out}", flush=True)
+            return out
+        finally:
+            fcntl.flock(lk.fileno(), fcntl.LOCK_UN)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("-j", "--jobs", type=int, default=int(os.environ.get("MAX_JOBS", "8")))
     ap.add_argument("--force", action="store_true")
+    ap.add_argument("--seqmix", action="store_true",
+                    help="build only the sequence-mixing kernel library (lumen/_C_seqmix.so)")
     a = ap.parse_args()
-    build(jobs=a.jobs, force=a.force)
+    if not a.seqmix:
+        build(jobs=a.jobs, force=a.force)
+    build_seqmix(jobs=a.jobs, force=a.force)
 
 
 if __name__ == "__main__":

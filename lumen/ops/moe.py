@@ -17,7 +17,8 @@ import torch.nn.functional as F
 
 
 def route_topk_ref(z: torch.Tensor, top: int) -> torch.Tensor:
-    val, idx = torch.topk(z.float(), top, -1)
+    val, idx = torch.sort(z.float(), dim=-1, descending=True, stable=True)  # ties: lowest index
+    val, idx = val[:, :top], idx[:, :top]
     return torch.zeros_like(z, dtype=torch.float32).scatter_(1, idx, torch.softmax(val, -1))
 
 
