@@ -490,6 +490,14 @@ def main():
                     help="(default, GPU) extra.box: clock / power sampled through the timed "
                          "region plus a fixed 8192^3 GEMM and a 4 GiB HBM read")
     ap.add_argument("--no_box", dest="box", action="store_false")
+    ap.add_argument("--hybrid", action="store_true",
+                    help="instead of the default workload: prefill / decode throughput of the "
+                         "hybrid design (Gedatar) beside Llama at equal size, one GPU "
+                         "(lumen/bench/hybrid_bench.py)")
+    ap.add_argument("--hybrid_widths", default="2048,4096")
+    ap.add_argument("--hybrid_batch", default="8,64", help="sequences per step (comma list)")
+    ap.add_argument("--hybrid_prompt", type=int, default=512)
+    ap.add_argument("--hybrid_decode_steps", type=int, default=32)
     args = ap.parse_args()
 
     import torch
@@ -507,6 +515,12 @@ def main():
 
         nat._C, nat._err = None, None
         assert nat.native() is not None, nat.native_error()
+
+    if args.hybrid:
+        from lumen.bench.hybrid_bench import run_hybrid_bench
+
+        run_hybrid_bench(args)
+        return
 
     from lumen.lora import LoraConfig, apply_lora, count_parameters
     from lumen.models import build_model, get_config

@@ -1,0 +1,137 @@
+"""Prefill / decode throughput of the hybrid design (Gedatar) beside Llama at equal size.
+
+``python bench.py --hybrid`` (one GPU).  Both models get random weights of layer shapes that
+resemble real models (width 2048 / 4096, head size 128 / 64, FFN 2.75 x width, vocab 32000), the
+same depth, and run the same forced-token workload through the serving engine
+(``lumen.serve.trace.TraceReplay``: the engine's input builder, block manager, state slots,
+runner, hipGraph decode):
+
+* prefill: ``--hybrid_batch`` prompts of ``--hybrid_prompt`` tokens in ONE step (tokens / s);
+* decode: one token for each of the sequences per step, ``--hybrid_decode_steps`` steps at that
+  context (tokens / s; the steps replay a decode graph).
+
+Prints one JSON line per (size, model) and a closing summary line.  Random weights, synthetic
+tokens; dtype bf16.
+"""
+from __future__ import annotations
+
+import json
+import time
+
+import torch
+
+
+def gedatar_config(width: int, depth_groups: int = 1):
+    from ..models.config import ModelConfig
+
+    W = width
+    ff = int(2.75 * W)
+    att = lambda mlp: {"type": "attention", "mlp": mlp,  # noqa: E731
+                       "mixer": {"heads": W // 128, "kv_heads": max(1, W // 512), "dim": 128,
+                                 "vdim": 128, "scale": 0.09, "mask": {"size": 1024}}}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": ff // 4},
+           "shared": {"ff": ff // 4}}
+    layers = [att(dense), {"type": "wkv", "mixer": {"heads": W // 64, "dim": 64}, "mlp": moe},
+              {"type": "general_delta", "mixer": {"heads": W // 128, "dim": 128}, "mlp": dense},
+              att(moe)] * depth_groups
+    return ModelConfig(arch="gedatar", vocab_size=32000, hidden_size=W,
+                       num_hidden_layers=len(layers), rms_norm_eps=1e-6, canon_taps=4,
+                       intermediate_size=0, num_attention_heads=0, num_key_value_heads=0,
+                       max_position_embeddings=1 << 20, eos_token_id=-1,
+                       name=f"gedatar-w{W}", layer_specs=layers)
+
+
+def llama_config(width: int, layers: int):
+    from ..models.config import ModelConfig
+
+    return ModelConfig(arch="llama", vocab_size=32000, hidden_size=width,
+                       intermediate_size=int(2.75 * width), num_hidden_layers=layers,
+                       num_attention_heads=width // 128, num_key_value_heads=max(1, width // 512),
+                       max_position_embeddings=4096, name=f"llama-w{width}")
+
+
+def _timed(fn, dev) -> float:
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    fn()
+    torch.cuda.synchronize(dev)
+    return time.perf_counter() - t0
+
+
+def run_one(cfg, batch: int, prompt: int, decode_steps: int, warmup: int, dev) -> dict:
+    from ..models import build_model
+    from ..serve.engine import EngineConfig, LLMEngine
+    from ..serve.trace import TraceReplay
+
+    model = build_model(cfg, dtype=torch.bfloat16, device=dev, init="random", seed=0)
+    bs = 16
+    total = prompt + decode_steps + warmup + 2
+    blocks = batch * ((total + bs - 1) // bs) + 8
+
+    class _Tok:
+        eos_token_id = None
+
+    eng = LLMEngine(EngineConfig(model=cfg.name, dtype="bf16", max_model_len=total + bs,
+                                 block_size=bs, num_blocks=blocks, max_num_seqs=batch,
+                                 max_num_batched_tokens=batch * prompt, async_scheduling=False),
+                    model=model, tokenizer=_Tok())
+    rp = TraceReplay(eng)
+    g = torch.Generator().manual_seed(1)
+    ids = torch.randint(3, cfg.vocab_size, (batch, total), generator=g).tolist()
+    names = [f"s{i}" for i in range(batch)]
+
+    def prefill(tag):
+        return rp.step([{"id": tag + n, "tokens": ids[i][:prompt], "want": [prompt - 1]}
+                        for i, n in enumerate(names)], [])
+
+    # warm-up prefill on throw-away requests (GEMM heuristics, allocator), then the timed one
+    prefill("w")
+    for n in names:
+        rp._retire("w" + n)
+    t_pre = _timed(lambda: prefill(""), dev)
+
+    def decode(j):
+        return rp.step([{"id": n, "tokens": [ids[i][prompt + j]], "want": [0]}
+                        for i, n in enumerate(names)], [])
+
+    for j in range(warmup):
+        decode(j)
+    t_dec = _timed(lambda: [decode(warmup + j) for j in range(decode_steps)], dev)
+    out = {"model": cfg.name, "params_m": round(cfg.num_params() / 1e6, 1), "batch": batch,
+           "prompt": prompt, "prefill_tok_s": round(batch * prompt / t_pre, 1),
+           "prefill_ms": round(t_pre * 1e3, 3), "decode_steps": decode_steps,
+           "decode_tok_s": round(batch * decode_steps / t_dec, 1),
+           "decode_ms_per_step": round(t_dec / decode_steps * 1e3, 3)}
+    del rp, eng, model
+    torch.cuda.empty_cache()
+    return out
+
+
+def run_hybrid_bench(args) -> list:
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    from ..ops._native import native, native_error
+
+    assert native() is not None, native_error()
+    rows = []
+    for width in [int(w) for w in str(args.hybrid_widths).split(",")]:
+        gcfg = gedatar_config(width)
+        for cfg in (gcfg, llama_config(width, gcfg.num_hidden_layers)):
+            for batch in [int(b) for b in str(args.hybrid_batch).split(",")]:
+                r = run_one(cfg, batch, args.hybrid_prompt, args.hybrid_decode_steps, 3, dev)
+                r["width"] = width
+                rows.append(r)
+                print(json.dumps(r), flush=True)
+    by = {(r["width"], r["batch"], r["model"].split("-")[0]): r for r in rows}
+    summ = []
+    for (w, b, kind), r in by.items():
+        if kind != "gedatar":
+            continue
+        ll = by[(w, b, "llama")]
+        summ.append({"width": w, "batch": b,
+                     "prefill_vs_llama": round(r["prefill_tok_s"] / ll["prefill_tok_s"], 3),
+                     "decode_vs_llama": round(r["decode_tok_s"] / ll["decode_tok_s"], 3)})
+    print(json.dumps({"metric": "hybrid_vs_llama_tokens_per_s", "dtype": "bf16",
+                      "data": "synthetic", "rows": summ}), flush=True)
+    return rows

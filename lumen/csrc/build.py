@@ -146,7 +146,9 @@ def _build_locked(jobs, force, verbose, build_dir, out) -> str:
         obj = os.path.join(build_dir, os.path.basename(src) + ".o")
         objs.append(obj)
         if force or _newer([src] + headers, obj):
-            cmd = [HIPCC, f"--offload-arch={ARCH}", "-munsafe-fp-atomics", *common, "-c", src,
+            # no packed-fp32 instructions (v_pk_*_f32): scalar fp32 code only
+            cmd = [HIPCC, f"--offload-arch={ARCH}", "-munsafe-fp-atomics", "-Xclang",
+                   "-target-feature", "-Xclang", "-packed-fp32-ops", *common, "-c", src,
                    "-o", obj]
             jobs_list.append(cmd)
     cpu_src = os.path.join(HERE, "cpu", "cpu_adam.cpp")

@@ -104,9 +104,236 @@ chunk_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ 
   }
 }
 
+// ---- prefill tiles on the matrix cores (16-bit dtypes, D a multiple of 32) ---------------------
+// A workgroup of NW waves takes 32 * NW consecutive rows of ONE segment and one query head; the
+// keys the tile can see (from the first row's chunk start to the last row's position) are
+// visited 32 at a time, staged in LDS twice (row-major for the scores, transposed for the value
+// pass) and shared by the waves.  Per wave (32 queries) and key tile, with v_mfma_f32_32x32x16:
+//   S^T = K Q^T      keys on the accumulator rows, queries on the columns (lane & 31): a lane
+//                    owns ONE query, so its running max / sum / correction are plain scalars;
+//                    q and k enter un-normalised (exactly as projected) and the two RMS factors
+//                    multiply the fp32 score (k's sum of squares comes from the operand the lane
+//                    loads anyway);
+//   O^T += V^T P^T   the accumulator registers 8s .. 8s+7 of S^T are keys {16s + 4hi + 0..3,
+//                    16s + 8 + 4hi + 0..3}: exactly one k = 16 operand when the transposed key
+//                    image is read in that order, so P goes from registers to the next product
+//                    without touching LDS.  P is split into a 16-bit head and a 16-bit remainder
+//                    (two products), which keeps ~16 mantissa bits of the fp32 weights.
+// Accumulator layout of the 32x32 products: lane l, register 4j + i = row 8j + 4(l >> 5) + i,
+// column l & 31; operand lanes hold k = 8(l >> 5) + 0..7.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8v __attribute__((ext_vector_type(8)));
+
+template <typename T> struct Mma32;
+template <> struct Mma32<bf16> {
+  static __device__ __forceinline__ f32x16 run(uint4 a, uint4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8v, a),
+                                                   __builtin_bit_cast(bf16x8v, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma32<fp16> {
+  static __device__ __forceinline__ f32x16 run(uint4 a, uint4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8v, a),
+                                                  __builtin_bit_cast(f16x8v, b), c, 0, 0, 0);
+  }
+};
+
+template <typename T>
+__device__ __forceinline__ float sumsq8(uint4 v) {
+  const T* e = reinterpret_cast<const T*>(&v);
+  float s = 0.f;
+#pragma unroll
+  for (int x = 0; x < 8; ++x) { const float f = to_f32(e[x]); s += f * f; }
+  return s;
+}
+
+template <typename T, int D, int NW>
+__global__ void __launch_bounds__(64 * NW)
+tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ cache,
+                 T* __restrict__ out, const int* __restrict__ tables, int maxb,
+                 const int* __restrict__ tiles, const int* __restrict__ cu,
+                 const int* __restrict__ start, int H, int G, int bs, float scale, float eps,
+                 int chunk, int sink) {
+  constexpr int QT = 32 * NW, LK = D + 8, LT = 40, NV = D / 8;
+  __shared__ __align__(16) T s_k[32 * LK];    // key tile, row-major
+  __shared__ __align__(16) T s_t[D * LT];     // key tile, transposed [d][key]
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c = lane & 31, hi = lane >> 5;
+  const int hd = blockIdx.y, g = hd / (H / G);
+  const int sg = tiles[2 * blockIdx.x], row0 = tiles[2 * blockIdx.x + 1];
+  const int seg_r0 = cu[sg], p0 = start[sg];
+  const int nrows = min(QT, cu[sg + 1] - row0);
+  const int* tbl = tables + (long long)sg * maxb;
+
+  const bool qv = 32 * w + c < nrows;
+  const int qrow = row0 + 32 * w + c;
+  const int pos = qv ? p0 + (qrow - seg_r0) : -1;
+  const int lo = (chunk > 0 && qv) ? (pos / chunk) * chunk : 0;
+  uint4 qreg[D / 16];
+  float q2 = 0.f;
+#pragma unroll
+  for (int kk = 0; kk < D / 16; ++kk) {
+    qreg[kk] = qv ? *reinterpret_cast<const uint4*>(q + (long long)qrow * ldq + hd * D + 16 * kk + 8 * hi)
+                  : make_uint4(0, 0, 0, 0);
+    q2 += sumsq8<T>(qreg[kk]);
+  }
+  q2 += __shfl_xor(q2, 32, 64);
+  const float qn = scale / sqrtf(q2 / D + eps);
+
+  const int pos_first = p0 + (row0 - seg_r0), kend = pos_first + nrows - 1;
+  const int kbeg = chunk > 0 ? (pos_first / chunk) * chunk : 0;
+  const bool wave_on = 32 * w < nrows;
+  const int wpos_min = pos_first + 32 * w, wpos_max = min(kend, wpos_min + 31);
+  const int wlo_min = chunk > 0 ? (wpos_min / chunk) * chunk : 0;
+
+  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  f32x16 O[D / 32];
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) O[db][r] = 0.f;
+
+  for (int k0 = kbeg; k0 <= kend; k0 += 32) {
+    __syncthreads();                       // the previous tile has been consumed
+    for (int idx = tid; idx < 32 * NV; idx += 64 * NW) {
+      const int key = idx / NV, part = idx % NV, j = k0 + key;
+      uint4 val = make_uint4(0, 0, 0, 0);
+      if (j <= kend) {
+        const long long off = (((long long)tbl[j / bs] * bs + j % bs) * G + g) * D;
+        val = *reinterpret_cast<const uint4*>(cache + off + 8 * part);
+      }
+      *reinterpret_cast<uint4*>(&s_k[key * LK + 8 * part]) = val;
+      const T* e = reinterpret_cast<const T*>(&val);
+#pragma unroll
+      for (int x = 0; x < 8; ++x) s_t[(8 * part + x) * LT + key] = e[x];
+    }
+    __syncthreads();
+    if (!wave_on || k0 > wpos_max || k0 + 31 < wlo_min) continue;   // nothing this wave may see
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    float k2 = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < D / 16; ++kk) {
+      const uint4 a = *reinterpret_cast<const uint4*>(&s_k[c * LK + 16 * kk + 8 * hi]);
+      k2 += sumsq8<T>(a);
+      acc = Mma32<T>::run(a, qreg[kk], acc);
+    }
+    k2 += __shfl_xor(k2, 32, 64);
+    const float kn = 1.f / sqrtf(k2 / D + eps);          // of key k0 + c
+
+    float sc[16];
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int keyr = 8 * (r >> 2) + 4 * hi + (r & 3);
+      const int j = k0 + keyr;
+      const float knr = __shfl(kn, keyr, 64);
+      const bool ok = j >= lo && j <= pos;
+      sc[r] = ok ? acc[r] * qn * knr : -INFINITY;
+      mloc = fmaxf(mloc, sc[r]);
+    }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+    const float mn = fmaxf(m, mloc);
+    const float ms = mn == -INFINITY ? 0.f : mn;
+    const float corr = expf(m - ms);
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { sc[r] = expf(sc[r] - ms); psum += sc[r]; }
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = mn;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) O[db][r] *= corr;
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      unsigned ph[4], pl[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const float a0 = sc[8 * s2 + 2 * x], a1 = sc[8 * s2 + 2 * x + 1];
+        const float h0 = to_f32(from_f32<T>(a0)), h1 = to_f32(from_f32<T>(a1));
+        ph[x] = pk2<T>(a0, a1);
+        pl[x] = pk2<T>(a0 - h0, a1 - h1);
+      }
+      const uint4 bh = make_uint4(ph[0], ph[1], ph[2], ph[3]);
+      const uint4 bl = make_uint4(pl[0], pl[1], pl[2], pl[3]);
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db) {
+        const T* tp = &s_t[(32 * db + c) * LT + 16 * s2 + 4 * hi];
+        const uint2 a0 = *reinterpret_cast<const uint2*>(tp);
+        const uint2 a1 = *reinterpret_cast<const uint2*>(tp + 8);
+        const uint4 a = make_uint4(a0.x, a0.y, a1.x, a1.y);
+        O[db] = Mma32<T>::run(a, bh, O[db]);
+        O[db] = Mma32<T>::run(a, bl, O[db]);
+      }
+    }
+  }
+  if (qv) {
+    const float inv = 1.f / l;
+    T* op = out + ((long long)qrow * H + hd) * D;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = 32 * db + 8 * j + 4 * hi;
+        const unsigned x0 = pk2<T>(O[db][4 * j] * inv, O[db][4 * j + 1] * inv);
+        const unsigned x1 = pk2<T>(O[db][4 * j + 2] * inv, O[db][4 * j + 3] * inv);
+        *reinterpret_cast<uint2*>(op + d) = make_uint2(x0, x1);
+      }
+  }
+}
+
+template <typename T>
+hipError_t launch_tiles(const void* q, long long ldq, const void* cache, void* out,
+                        const int* tables, int maxb, const int* tiles, int ntiles, const int* cu,
+                        const int* start, int H, int G, int D, int bs, float scale, float eps,
+                        int chunk, int sink, hipStream_t st) {
+  const dim3 grid(ntiles, H);
+#define GO(DD)                                                                                  \
+  tile_attn_kernel<T, DD, 2><<<grid, 128, 0, st>>>((const T*)q, ldq, (const T*)cache, (T*)out,  \
+                                                   tables, maxb, tiles, cu, start, H, G, bs,    \
+                                                   scale, eps, chunk, sink)
+  switch (D) {
+    case 32: GO(32); break;
+    case 64: GO(64); break;
+    case 96: GO(96); break;
+    case 128: GO(128); break;
+    case 192: GO(192); break;
+    case 256: GO(256); break;
+    default: return hipErrorInvalidValue;
+  }
+#undef GO
+  return hipGetLastError();
+}
+
 }  // namespace
 
 extern "C" {
+
+// 1 when sm_chunk_attn_tiles has a kernel for this dtype / head size
+int sm_chunk_attn_tiles_ok(int dt, int D) {
+  return (dt == kBF16 || dt == kF16) &&
+         (D == 32 || D == 64 || D == 96 || D == 128 || D == 192 || D == 256);
+}
+
+// tiles: [ntiles, 2] int32 (segment, first row); every tile covers up to 64 rows of its segment
+hipError_t sm_chunk_attn_tiles(int dt, const void* q, long long ldq, const void* cache, void* out,
+                               const int* tables, int maxb, const int* tiles, int ntiles,
+                               const int* cu, const int* start, int H, int G, int D, int bs,
+                               float scale, float eps, int chunk, int sink, hipStream_t st) {
+  if (ntiles == 0) return hipSuccess;
+  if (G < 1 || H % G || bs < 1 || chunk < 0 || (ldq % 8) != 0) return hipErrorInvalidValue;
+  if (dt == kBF16)
+    return launch_tiles<bf16>(q, ldq, cache, out, tables, maxb, tiles, ntiles, cu, start, H, G, D,
+                              bs, scale, eps, chunk, sink, st);
+  if (dt == kF16)
+    return launch_tiles<fp16>(q, ldq, cache, out, tables, maxb, tiles, ntiles, cu, start, H, G, D,
+                              bs, scale, eps, chunk, sink, st);
+  return hipErrorInvalidValue;
+}
 
 hipError_t sm_chunk_attn(int dt, const void* q, long long ldq, const void* cache, void* out,
                          const int* tables, int maxb, const int* row_seg, const int* positions,

@@ -30,6 +30,7 @@ SIGNATURES = {
     "sm_gdelta": "iplplplplplplppppplpppiiifff",
     "sm_write_k": "iplppii",
     "sm_chunk_attn": "iplpppippiiiiiffii",
+    "sm_chunk_attn_tiles": "iplpppipippiiiiffii",
     "sm_route_topk": "ppiii",
     "sm_gated_act": "ipppiiii",
 }
@@ -50,6 +51,8 @@ def _load():
             fn = getattr(lib, name)
             fn.argtypes = [_T[c] for c in sig] + [ctypes.c_void_p]
             fn.restype = ctypes.c_int
+        lib.sm_chunk_attn_tiles_ok.argtypes = [ctypes.c_int, ctypes.c_int]
+        lib.sm_chunk_attn_tiles_ok.restype = ctypes.c_int
         _lib = lib
     except Exception as e:  # pragma: no cover - depends on build state
         _err = e
@@ -72,6 +75,11 @@ def use_seqmix(t: torch.Tensor) -> bool:
 
 
 DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def tiles_ok(dt: int, D: int) -> bool:
+    """Does the matrix-core prefill attention have a kernel for this dtype code / head size?"""
+    return bool(_load().sm_chunk_attn_tiles_ok(dt, D))
 
 
 def _arg(kind, v):

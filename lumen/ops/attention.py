@@ -555,7 +555,7 @@ def chunk_sink_attention(q: torch.Tensor, cache: torch.Tensor, seg, H: int, G: i
                          scale: float, chunk: int, eps: float, sink: bool = True) -> torch.Tensor:
     """q [T, H * D] (rows may be strided) against the paged raw-key cache; the step's own keys
     must already be in the cache (``write_key_cache``).  Returns [T, H * D] in q's dtype."""
-    from ._seqmix import DT, call, use_seqmix
+    from ._seqmix import DT, call, tiles_ok, use_seqmix
 
     if not use_seqmix(q):
         return chunk_sink_attention_ref(q, cache, seg, H, G, D, scale, chunk, eps, sink)
@@ -565,7 +565,18 @@ def chunk_sink_attention(q: torch.Tensor, cache: torch.Tensor, seg, H: int, G: i
         raise ValueError(f"attention head size {D} > 256 is not supported")
     T = q.shape[0]
     out = torch.empty(T, H * D, dtype=q.dtype, device=q.device)
-    call("sm_chunk_attn", DT[q.dtype], q, q.stride(0), cache, out, seg.tables,
-         seg.tables.shape[1], seg.row_seg, seg.positions, T, H, G, D, cache.shape[1], scale, eps,
-         chunk, int(sink))
+    maxb, bs = seg.tables.shape[1], cache.shape[1]
+    # prefill chunks: 64-row tiles on the matrix cores (16-bit dtypes, head sizes it is built
+    # for); decode rows, fp32 and other head sizes: one wave per (row, head)
+    Tp = 0
+    if (seg.q_tiles is not None and seg.tile_rows > 0 and q.stride(0) % 8 == 0
+            and q.data_ptr() % 16 == 0 and tiles_ok(DT[q.dtype], D)):
+        Tp = seg.tile_rows
+        call("sm_chunk_attn_tiles", DT[q.dtype], q, q.stride(0), cache, out, seg.tables, maxb,
+             seg.q_tiles, seg.q_tiles.shape[0], seg.cu, seg.start, H, G, D, bs, scale, eps, chunk,
+             int(sink))
+    if T > Tp:
+        call("sm_chunk_attn", DT[q.dtype], q[Tp:], q.stride(0), cache, out[Tp:], seg.tables, maxb,
+             seg.row_seg[Tp:], seg.positions[Tp:], T - Tp, H, G, D, bs, scale, eps, chunk,
+             int(sink))
     return out

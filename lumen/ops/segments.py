@@ -21,6 +21,11 @@ class SegBatch:
     positions: torch.Tensor   # [T] int32 position of each row in its sequence
     tables: Optional[torch.Tensor] = None   # [S, max_blocks] int32 cache blocks per segment
     cache_slots: Optional[torch.Tensor] = None  # [T] int64 cache slot of each row (-1: none)
+    # prefill rows cut into tiles for the matrix-core attention kernel: [n, 2] int32 (segment,
+    # first row), each tile up to TILE_ROWS rows of its segment; they cover rows [0, tile_rows)
+    # (the prefill chunks; decode rows follow and take the row kernel).  None: row kernel only.
+    q_tiles: Optional[torch.Tensor] = None
+    tile_rows: int = 0
 
     @property
     def S(self) -> int:
@@ -29,6 +34,15 @@ class SegBatch:
     @property
     def T(self) -> int:
         return self.row_seg.shape[0]
+
+
+TILE_ROWS = 64
+
+
+def tile_list(cu, n_segments: int):
+    """[(segment, first row)] covering the first ``n_segments`` segments of row offsets ``cu``
+    (host ints) in tiles of TILE_ROWS rows."""
+    return [(s, r) for s in range(n_segments) for r in range(int(cu[s]), int(cu[s + 1]), TILE_ROWS)]
 
 
 def whole_sequences(lengths, device, slots=None, block_size: int = 16) -> SegBatch:
@@ -51,4 +65,5 @@ def whole_sequences(lengths, device, slots=None, block_size: int = 16) -> SegBat
         b0 += nb[i]
     return SegBatch(torch.tensor(cu, **i32),
                     torch.tensor(list(slots) if slots is not None else list(range(S)), **i32),
-                    torch.zeros(S, **i32), row_seg, pos, tables, torch.cat(cache_slots))
+                    torch.zeros(S, **i32), row_seg, pos, tables, torch.cat(cache_slots),
+                    torch.tensor(tile_list(cu, S), **i32).view(-1, 2), cu[-1])

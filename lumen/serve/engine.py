@@ -429,8 +429,11 @@ class LLMEngine:
                 seg_tbl[i, :len(t)] = t
             if N:
                 seg_tbl[P:, :maxb_d] = dec_bt
+            from ..ops.segments import tile_list
+
+            tiles = np.asarray(tile_list(seg_cu, P), dtype=np.int64).reshape(-1)
             seg_arrays = [seg_cu, seg_slot, seg_start, np.repeat(np.arange(S), lens_s),
-                          seg_tbl.reshape(-1)]
+                          seg_tbl.reshape(-1), tiles]
             seg_n = sum(a.size for a in seg_arrays)
             extra += seg_arrays
         host = np.concatenate([np.concatenate(parts)] + extra)
@@ -475,9 +478,11 @@ class LLMEngine:
             from ..ops.segments import SegBatch
 
             g = dev[o:o + seg_n].int()
+            t0 = 3 * S + 1 + T + S * maxb
             inp.seg = SegBatch(g[:S + 1], g[S + 1:2 * S + 1], g[2 * S + 1:3 * S + 1],
                                g[3 * S + 1:3 * S + 1 + T], inp.positions,
-                               g[3 * S + 1 + T:].view(S, maxb), inp.slots)
+                               g[3 * S + 1 + T:t0].view(S, maxb), inp.slots,
+                               g[t0:].view(-1, 2) if Tp else None, Tp)
         return inp
 
     def _to_device(self, host: "np.ndarray") -> torch.Tensor:

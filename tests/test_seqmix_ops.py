@@ -1,6 +1,8 @@
-"""The sequence-mixing HIP kernels (lumen/csrc/seqmix) against the float64 oracle of
-tests/_ref_gedatar.py, one mechanism at a time, on steps cut into segments: whole sequences,
-pieces down to two tokens and single rows, state slots and cache blocks in scrambled order."""
+"""The sequence-mixing ops against the float64 oracle of tests/_ref_gedatar.py, one mechanism at
+a time, on steps cut into segments: whole sequences, pieces down to two tokens and single rows,
+state slots holding stale values and cache blocks in scrambled order.  The HIP kernels
+(lumen/csrc/seqmix) run every case (marked ``gpu``); the ops' torch path, which the CPU engine
+uses, runs the mixed-pieces fp32 case of each."""
 import math
 
 import pytest
@@ -9,10 +11,18 @@ import torch
 from _ref_gedatar import (F64, ref_attention, ref_canon, ref_delta, ref_dyt, ref_route,
                           ref_token_shift, ref_unit_rms, ref_wkv)
 
-pytestmark = pytest.mark.gpu
-
 DEV = "cuda"
 DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(autouse=True)
+def _device(request):
+    """Tests whose parameters start with the device run there; all others on the GPU."""
+    global DEV
+    DEV = request.node.callspec.params.get("dev", "cuda") if hasattr(request.node, "callspec") \
+        else "cuda"
+    yield
+    DEV = "cuda"
 
 
 def tol(dtype):
@@ -38,8 +48,8 @@ def cut_steps(lengths, pieces, seed):
             yield step
 
 
-def seg_of(step, slots, tables=None, bs=16):
-    from lumen.ops.segments import SegBatch
+def seg_of(step, slots, tables=None, bs=16, tiled=False):
+    from lumen.ops.segments import SegBatch, tile_list
 
     i32 = dict(dtype=torch.int32, device=DEV)
     cu, row_seg, pos, cs = [0], [], [], []
@@ -53,10 +63,14 @@ def seg_of(step, slots, tables=None, bs=16):
     if tables is not None:
         mb = max(len(t) for t in tables)
         tb = torch.tensor([tables[s] + [0] * (mb - len(tables[s])) for s, _, _ in step], **i32)
-    return SegBatch(torch.tensor(cu, **i32), torch.tensor([slots[s] for s, _, _ in step], **i32),
-                    torch.tensor([lo for _, lo, _ in step], **i32), torch.tensor(row_seg, **i32),
-                    torch.tensor(pos, **i32), tb,
-                    torch.tensor(cs, dtype=torch.long, device=DEV) if tables is not None else None)
+    sb = SegBatch(torch.tensor(cu, **i32), torch.tensor([slots[s] for s, _, _ in step], **i32),
+                  torch.tensor([lo for _, lo, _ in step], **i32), torch.tensor(row_seg, **i32),
+                  torch.tensor(pos, **i32), tb,
+                  torch.tensor(cs, dtype=torch.long, device=DEV) if tables is not None else None)
+    if tiled:       # every segment through the matrix-core tiles (where the op has them)
+        sb.q_tiles = torch.tensor(tile_list(cu, len(step)), **i32).view(-1, 2)
+        sb.tile_rows = cu[-1]
+    return sb
 
 
 def gather(step, per_seq):
@@ -73,12 +87,17 @@ def scatter(step, rows, outs):
 LENGTHS = [37, 5, 70, 2]
 SLOTS = [3, 0, 5, 1]
 PIECES = [[1000], [7, 2, 1, 16, 3], [1], [2]]
+GPU = pytest.mark.gpu
+# (device, dtype, pieces): every combination on the GPU, one on the CPU path
+CASES = [pytest.param("cuda", d, p, marks=GPU, id=f"cuda-{str(d)[6:]}-{i}")
+         for d in DTYPES for i, p in enumerate(PIECES)] + [
+    pytest.param("cpu", torch.float32, PIECES[1], id="cpu-float32-1")]
+DEVS = ["cpu", pytest.param("cuda", marks=GPU)]
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("pieces", PIECES)
+@pytest.mark.parametrize("dev,dtype,pieces", CASES)
 @pytest.mark.parametrize("taps", [1, 2, 4])
-def test_dyt_canon_segments(dtype, pieces, taps):
+def test_dyt_canon_segments(dev, dtype, pieces, taps):
     from lumen.ops.conv import dyt_canon
 
     torch.manual_seed(taps)
@@ -97,8 +116,9 @@ def test_dyt_canon_segments(dtype, pieces, taps):
         torch.testing.assert_close(g, r, **tol(dtype))
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_dyt_and_residual(dtype):
+@pytest.mark.parametrize("dev,dtype", [("cpu", torch.float32)] + [
+    pytest.param("cuda", d, marks=GPU) for d in DTYPES])
+def test_dyt_and_residual(dev, dtype):
     from lumen.ops.norm import dyt, dyt_residual
 
     torch.manual_seed(0)
@@ -119,9 +139,8 @@ def test_dyt_and_residual(dtype):
                                ref_dyt(x.to(F64), *r64(n2)), **tol(dtype))
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("pieces", PIECES)
-def test_token_shift_segments(dtype, pieces):
+@pytest.mark.parametrize("dev,dtype,pieces", CASES)
+def test_token_shift_segments(dev, dtype, pieces):
     from lumen.ops.recurrent import token_shift
 
     torch.manual_seed(2)
@@ -147,10 +166,9 @@ def _scan_inputs(H, D, dtype, seed, n_in):
     return [[mk(n, 0.7) for _ in range(n_in)] for n in LENGTHS], g
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("pieces", PIECES)
+@pytest.mark.parametrize("dev,dtype,pieces", CASES)
 @pytest.mark.parametrize("H,D", [(2, 32), (3, 48), (1, 64), (2, 80)])
-def test_wkv_scan_segments(dtype, pieces, H, D):
+def test_wkv_scan_segments(dev, dtype, pieces, H, D):
     from lumen.ops.recurrent import wkv_scan
 
     ins, g = _scan_inputs(H, D, dtype, D, 5)         # r k v wl gate
@@ -175,10 +193,9 @@ def test_wkv_scan_segments(dtype, pieces, H, D):
         torch.testing.assert_close(gg, r, **tol(dtype))
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("pieces", PIECES)
+@pytest.mark.parametrize("dev,dtype,pieces", CASES)
 @pytest.mark.parametrize("H,D", [(2, 32), (3, 48), (1, 128)])
-def test_delta_scan_segments(dtype, pieces, H, D):
+def test_delta_scan_segments(dev, dtype, pieces, H, D):
     from lumen.ops.recurrent import delta_scan
 
     ins, g = _scan_inputs(H, D, dtype, D + 1, 6)     # r k v wl al gl
@@ -204,6 +221,7 @@ def test_delta_scan_segments(dtype, pieces, H, D):
         torch.testing.assert_close(gg, r, **tol(dtype))
 
 
+@pytest.mark.gpu
 def test_scan_strided_inputs_match_contiguous():
     """Column slices of one fused projection (row stride > H * D) give the same result."""
     from lumen.ops.recurrent import wkv_scan
@@ -221,11 +239,10 @@ def test_scan_strided_inputs_match_contiguous():
     assert torch.equal(outs[0], outs[1])
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("pieces", PIECES)
+@pytest.mark.parametrize("dev,dtype,pieces", CASES)
 @pytest.mark.parametrize("H,G,D,chunk,bs", [(4, 2, 32, 24, 16), (2, 2, 64, 16, 16),
                                              (6, 1, 40, 33, 8), (3, 3, 20, 0, 16)])
-def test_chunk_sink_attention_segments(dtype, pieces, H, G, D, chunk, bs):
+def test_chunk_sink_attention_segments(dev, dtype, pieces, H, G, D, chunk, bs):
     from lumen.ops.attention import chunk_sink_attention, write_key_cache
 
     torch.manual_seed(H * D + chunk)
@@ -245,7 +262,7 @@ def test_chunk_sink_attention_segments(dtype, pieces, H, G, D, chunk, bs):
     cache = torch.full((nb + 3, bs, G, D), 50.0, device=DEV, dtype=dtype)
     got = [torch.zeros(n, H * D, dtype=F64) for n in LENGTHS]
     for step in cut_steps(LENGTHS, pieces, 5):
-        sg = seg_of(step, SLOTS, tables, bs)
+        sg = seg_of(step, SLOTS, tables, bs, tiled=(H + chunk) % 2 == 0)
         write_key_cache(gather(step, ks).to(DEV), cache, sg.cache_slots)
         out = chunk_sink_attention(gather(step, qs).to(DEV), cache, sg, H, G, D, scale, chunk, eps)
         scatter(step, out, got)
@@ -253,7 +270,9 @@ def test_chunk_sink_attention_segments(dtype, pieces, H, G, D, chunk, bs):
         torch.testing.assert_close(gg, r, **tol(dtype))
 
 
-def test_attention_chunk_edges_and_sink_show():
+@pytest.mark.parametrize("dev", DEVS)
+@pytest.mark.parametrize("pieces", [[1000], [1], [3, 1, 2]])
+def test_attention_chunk_edges_and_sink_show(dev, pieces):
     """One key per chunk is made to dominate (an aligned query / key pair among small random
     ones), so a mask that is one position off, or a missing sink, moves the output by far more
     than the tolerance: the kernel must match the oracle and differ from both wrong variants."""
@@ -272,9 +291,13 @@ def test_attention_chunk_edges_and_sink_show():
     q64, k64 = q.to(F64).view(T, 1, D), k.to(F64).view(T, 1, D)
     ref = ref_attention(q64, k64, scale, chunk, 1e-6).view(T, D)
     cache = torch.zeros(4, bs, 1, D, device=DEV)
-    sg = seg_of([(0, 0, T)], [0], [[2, 0, 3]], bs)
-    write_key_cache(k.to(DEV), cache, sg.cache_slots)
-    out = chunk_sink_attention(q.to(DEV), cache, sg, H, G, D, scale, chunk, 1e-6).cpu().to(F64)
+    got = [torch.zeros(T, D, dtype=F64)]
+    for step in cut_steps([T], pieces, 0):   # prompt rows and decoded rows, chunk edges at and
+        sg = seg_of(step, [0], [[2, 0, 3]], bs)   # between block borders (chunk 8, blocks of 16)
+        write_key_cache(gather(step, [k]).to(DEV), cache, sg.cache_slots)
+        scatter(step, chunk_sink_attention(gather(step, [q]).to(DEV), cache, sg, H, G, D, scale,
+                                           chunk, 1e-6), got)
+    out = got[0]
     torch.testing.assert_close(out, ref, rtol=1e-5, atol=1e-5)
     for wrong in (ref_attention(q64, k64, scale, chunk + 1, 1e-6),
                   ref_attention(q64, k64, scale, chunk - 1, 1e-6),
@@ -283,8 +306,9 @@ def test_attention_chunk_edges_and_sink_show():
         assert float((wrong.view(T, D) - ref).abs().max()) > 0.05
 
 
+@pytest.mark.parametrize("dev", DEVS)
 @pytest.mark.parametrize("E,top", [(6, 3), (12, 2), (5, 1), (70, 4), (4, 4)])
-def test_route_topk(E, top):
+def test_route_topk(dev, E, top):
     from lumen.ops.moe import route_topk
 
     torch.manual_seed(E)
@@ -295,9 +319,10 @@ def test_route_topk(E, top):
     assert ((got > 0).sum(1) == top).all()
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dev,dtype", [("cpu", torch.float32)] + [
+    pytest.param("cuda", d, marks=GPU) for d in DTYPES])
 @pytest.mark.parametrize("E,ff,ffs", [(0, 0, 96), (5, 24, 40), (3, 16, 0)])
-def test_gated_act(dtype, E, ff, ffs):
+def test_gated_act(dev, dtype, E, ff, ffs):
     from lumen.ops.moe import gated_act
 
     torch.manual_seed(ff + ffs)
@@ -314,3 +339,104 @@ def test_gated_act(dtype, E, ff, ffs):
         parts.append(torch.nn.functional.silu(b[:, :ffs]) * b[:, ffs:])
     got = gated_act(gu.to(DEV), wts.to(DEV) if E else None, E, ff, ffs).cpu().to(F64)
     torch.testing.assert_close(got, torch.cat(parts, 1), **tol(dtype))
+
+
+@pytest.mark.parametrize("dev", DEVS)
+@pytest.mark.parametrize("kind", ["wkv", "delta"])
+@pytest.mark.parametrize("pieces", [[1000], [64, 1], [2]])
+def test_far_token_reaches_through_the_state(dev, kind, pieces):
+    """A write 250 tokens back, on slowly decaying channels, must still dominate the read-out: the
+    early token's key / value are large, a late query is aligned with that key.  A state that is
+    lost, reset or decayed by the wrong factor anywhere on the way changes the result by far more
+    than the tolerance (the oracle without the early token differs by > 0.5)."""
+    from lumen.ops.recurrent import delta_scan, wkv_scan
+
+    torch.manual_seed(7)
+    H, D, T, far, late = 2, 32, 260, 4, 255
+    mk = lambda s: torch.randn(T, H * D) * s  # noqa: E731
+    r, k, v, gl = mk(0.1), mk(0.1), mk(0.1), mk(1.0)
+    wl = torch.zeros(T, H * D)
+    al = torch.full((T, H * D), -6.0)                  # removal rate ~ 0
+    key = torch.zeros(H * D)
+    key[5], key[D + 9] = 4.0, 4.0
+    k[far] += key
+    v[far] += 3.0
+    r[late] += key
+    w0 = torch.full((H * D,), -7.0)                    # decay ~ 1 per step
+    u = torch.zeros(H * D)
+    ab = torch.zeros(H * D)
+    nw = torch.ones(H * D)
+    eps = 1e-6
+
+    def ref_of(k_, v_):
+        f = lambda t: t.to(F64).view(T, H, D)  # noqa: E731
+        if kind == "wkv":
+            w = torch.exp(-torch.exp(wl.to(F64) + w0.to(F64))).view(T, H, D)
+            o = ref_wkv(f(r), f(k_), f(v_), w, u.to(F64).view(H, D))
+            gate = torch.nn.functional.silu(gl.to(F64))
+        else:
+            w = torch.exp(-0.61 * torch.sigmoid(wl.to(F64) + w0.to(F64))).view(T, H, D)
+            o = ref_delta(f(r), f(k_), f(v_), w, torch.sigmoid(al.to(F64) + ab.to(F64)).view(T, H, D))
+            gate = torch.sigmoid(gl.to(F64))
+        return ref_unit_rms(o, eps).reshape(T, H * D) * gate
+
+    ref = ref_of(k, v)
+    k0, v0 = k.clone(), v.clone()
+    k0[far] -= key
+    v0[far] -= 3.0
+    assert float((ref_of(k0, v0)[late] - ref[late]).abs().max()) > 0.5
+    state = torch.full((3, H, D, D), 5.0, device=DEV)
+    got = [torch.zeros(T, H * D, dtype=F64)]
+    for step in cut_steps([T], pieces, 0):
+        a = [gather(step, [x]).to(DEV) for x in (r, k, v, wl, al, gl)]
+        sg = seg_of(step, [2])
+        if kind == "wkv":
+            out = wkv_scan(a[0], a[1], a[2], a[3], a[5], w0.to(DEV), u.to(DEV), nw.to(DEV), state,
+                           sg, H, D, eps)
+        else:
+            out = delta_scan(a[0], a[1], a[2], a[3], a[4], a[5], w0.to(DEV), ab.to(DEV),
+                             nw.to(DEV), state, sg, H, D, eps, 0.61, 1e-6)
+        scatter(step, out, got)
+    torch.testing.assert_close(got[0], ref, rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("pieces", [[1000], [64, 1, 70, 2, 33]])
+@pytest.mark.parametrize("H,G,D,chunk,bs", [(4, 2, 128, 48, 16), (2, 1, 96, 100, 16),
+                                             (3, 3, 32, 0, 8), (2, 2, 64, 5, 16),
+                                             (1, 1, 256, 64, 16), (2, 1, 192, 31, 4)])
+def test_tile_attention_matches_oracle(dtype, pieces, H, G, D, chunk, bs):
+    """The matrix-core prefill kernel: several 64-row tiles per segment, chunks that start inside
+    a tile, span tiles or are smaller than a key tile, segments that start mid-sequence; and the
+    row kernel on the same rows gives the same result to rounding."""
+    from lumen.ops.attention import chunk_sink_attention, write_key_cache
+
+    torch.manual_seed(D + chunk)
+    lengths, slots = [150, 33, 200], [0, 1, 2]
+    scale, eps = 0.6 / math.sqrt(D), 1e-5
+    qs = [(torch.randn(n, H * D) * 1.5).to(dtype) for n in lengths]
+    ks = [(torch.randn(n, G * D) * 1.5).to(dtype) for n in lengths]
+    ref = [ref_attention(q.to(F64).view(-1, H, D), k.to(F64).view(-1, G, D), scale, chunk, eps)
+           .reshape(-1, H * D) for q, k in zip(qs, ks)]
+    nb = sum((n + bs - 1) // bs for n in lengths)
+    perm = torch.randperm(nb + 2).tolist()
+    tables, at = [], 0
+    for n in lengths:
+        c = (n + bs - 1) // bs
+        tables.append(perm[at:at + c])
+        at += c
+    cache = torch.full((nb + 2, bs, G, D), 30.0, device=DEV, dtype=dtype)
+    got = [torch.zeros(n, H * D, dtype=F64) for n in lengths]
+    rows = [torch.zeros(n, H * D, dtype=F64) for n in lengths]
+    for step in cut_steps(lengths, pieces, 6):
+        sg = seg_of(step, slots, tables, bs, tiled=True)
+        write_key_cache(gather(step, ks).to(DEV), cache, sg.cache_slots)
+        qd = gather(step, qs).to(DEV)
+        scatter(step, chunk_sink_attention(qd, cache, sg, H, G, D, scale, chunk, eps), got)
+        sg.q_tiles, sg.tile_rows = None, 0
+        scatter(step, chunk_sink_attention(qd, cache, sg, H, G, D, scale, chunk, eps), rows)
+    t = dict(rtol=2e-2, atol=2e-2) if dtype == torch.bfloat16 else dict(rtol=3e-3, atol=3e-3)
+    for g_, r_, ref_ in zip(got, rows, ref):
+        torch.testing.assert_close(g_, ref_, **t)
+        torch.testing.assert_close(g_, r_, **t)
