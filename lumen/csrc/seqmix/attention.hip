@@ -193,21 +193,61 @@ tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ c
 #pragma unroll
     for (int r = 0; r < 16; ++r) O[db][r] = 0.f;
 
+  // staging: one item = 4 consecutive keys x 8 channels (four 16-byte loads); the row-major
+  // image takes them as they are, the transposed image takes eight 8-byte stores of 4 keys each
+  // (transposed in registers).  The next tile's loads are issued before this tile's products, so
+  // their latency hides behind the matrix work.
+  constexpr int NT = 64 * NW, ITEMS = (D + NT - 1) / NT;
+  uint4 pre[ITEMS][4];
+  auto prefetch = [&](int k0) {
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int item = tid + it * NT;
+      if (item < D) {
+        const int kq = item / NV, part = item % NV;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          const int j = k0 + 4 * kq + x;
+          pre[it][x] = make_uint4(0, 0, 0, 0);
+          if (j <= kend) {
+            const long long off = (((long long)tbl[j / bs] * bs + j % bs) * G + g) * D;
+            pre[it][x] = *reinterpret_cast<const uint4*>(cache + off + 8 * part);
+          }
+        }
+      }
+    }
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int item = tid + it * NT;
+      if (item < D) {
+        const int kq = item / NV, part = item % NV;
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+          *reinterpret_cast<uint4*>(&s_k[(4 * kq + x) * LK + 8 * part]) = pre[it][x];
+        const unsigned w0[4] = {pre[it][0].x, pre[it][0].y, pre[it][0].z, pre[it][0].w};
+        const unsigned w1[4] = {pre[it][1].x, pre[it][1].y, pre[it][1].z, pre[it][1].w};
+        const unsigned w2[4] = {pre[it][2].x, pre[it][2].y, pre[it][2].z, pre[it][2].w};
+        const unsigned w3[4] = {pre[it][3].x, pre[it][3].y, pre[it][3].z, pre[it][3].w};
+#pragma unroll
+        for (int mm = 0; mm < 4; ++mm) {     // word mm holds channels 2mm (low half), 2mm + 1
+          T* t0 = &s_t[(8 * part + 2 * mm) * LT + 4 * kq];
+          *reinterpret_cast<uint2*>(t0) = make_uint2((w0[mm] & 0xffffu) | (w1[mm] << 16),
+                                                     (w2[mm] & 0xffffu) | (w3[mm] << 16));
+          *reinterpret_cast<uint2*>(t0 + LT) = make_uint2(
+              (w0[mm] >> 16) | (w1[mm] & 0xffff0000u), (w2[mm] >> 16) | (w3[mm] & 0xffff0000u));
+        }
+      }
+    }
+  };
+
+  prefetch(kbeg);
   for (int k0 = kbeg; k0 <= kend; k0 += 32) {
     __syncthreads();                       // the previous tile has been consumed
-    for (int idx = tid; idx < 32 * NV; idx += 64 * NW) {
-      const int key = idx / NV, part = idx % NV, j = k0 + key;
-      uint4 val = make_uint4(0, 0, 0, 0);
-      if (j <= kend) {
-        const long long off = (((long long)tbl[j / bs] * bs + j % bs) * G + g) * D;
-        val = *reinterpret_cast<const uint4*>(cache + off + 8 * part);
-      }
-      *reinterpret_cast<uint4*>(&s_k[key * LK + 8 * part]) = val;
-      const T* e = reinterpret_cast<const T*>(&val);
-#pragma unroll
-      for (int x = 0; x < 8; ++x) s_t[(8 * part + x) * LT + key] = e[x];
-    }
+    commit();
     __syncthreads();
+    if (k0 + 32 <= kend) prefetch(k0 + 32);
     if (!wave_on || k0 > wpos_max || k0 + 31 < wlo_min) continue;   // nothing this wave may see
 
     f32x16 acc;

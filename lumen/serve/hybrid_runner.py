@@ -36,7 +36,7 @@ from ..models.config import ModelConfig
 from ..models.gedatar import DELTA_DECAY, DELTA_KEY_EPS
 from ..ops.attention import chunk_sink_attention, write_key_cache
 from ..ops.conv import dyt_canon
-from ..ops.moe import gated_act, route_topk
+from ..ops.moe import gated_act, moe, route_topk
 from ..ops.norm import dyt, dyt_residual
 from ..ops.recurrent import delta_scan, token_shift, wkv_scan
 from ..ops.segments import SegBatch, whole_sequences
@@ -194,13 +194,14 @@ def run_layers(w: HybridWeights, st: HybridState, tokens: torch.Tensor, seg: Seg
             x, _ = dyt_residual(x, y, L.norms["norm1b"], None, dt)
         else:
             x, h2 = dyt_residual(x, y, L.norms["norm1b"], L.norms["norm2"], dt)
-            wts = None
             if f["E"]:
                 # the router in fp32, on the (possibly 16-bit rounded) normed row
                 z = torch.addmm(f["router_b"], h2.float(), f["router"].t())
-                wts = route_topk(z, f["top"])
-            act = gated_act(F.linear(h2, f["gu"]), wts, f["E"], f["ff"], f["ffs"])
-            x, _ = dyt_residual(x, F.linear(act, f["down"]), L.norms["norm2b"], None, dt)
+                y2 = moe(h2, route_topk(z, f["top"]), f["gu"], f["down"], f["E"], f["top"],
+                         f["ff"], f["ffs"])
+            else:
+                y2 = F.linear(gated_act(F.linear(h2, f["gu"]), None, 0, 0, f["ffs"]), f["down"])
+            x, _ = dyt_residual(x, y2, L.norms["norm2b"], None, dt)
         if observe is not None:
             observe(i, x)
     return x

@@ -125,6 +125,17 @@ def test_whole_prompt_matches_oracle(device, name):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_prefill_step_large_enough_for_grouped_experts(device):
+    """A 300-row step runs the experts grouped by expert; cut into small steps (and decoding) the
+    same tokens run them through the all-experts form.  Both must be the oracle's logits."""
+    m = make("mixed4", device, seed=11)
+    toks = tokens(m, 300, 12)
+    ref = oracle(m).forward(toks)
+    check(replay_alone(m, device, toks, [1000]), ref)
+    check(replay_alone(m, device, toks, [128, 100, 1]), ref)
+
+
+@pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("name", list(CONFIGS))
 def test_prefill_then_long_decode(device, name):
     """A short prompt, then token by token across several chunk and block borders."""

@@ -440,3 +440,33 @@ def test_tile_attention_matches_oracle(dtype, pieces, H, G, D, chunk, bs):
     for g_, r_, ref_ in zip(got, rows, ref):
         torch.testing.assert_close(g_, ref_, **t)
         torch.testing.assert_close(g_, r_, **t)
+
+
+@pytest.mark.parametrize("dev", DEVS)
+@pytest.mark.parametrize("E,top,ff,ffs", [(6, 2, 24, 40), (4, 1, 16, 0), (5, 3, 8, 8)])
+def test_moe_dense_and_grouped_match_oracle(dev, E, top, ff, ffs):
+    """Both ways of running the experts (all experts with zero weights / each expert on its own
+    rows) against a per-expert loop; ``moe`` picks by step size."""
+    from lumen.ops import moe as M
+
+    torch.manual_seed(E * top)
+    T, W = 300, 64
+    h = torch.randn(T, W)
+    gu = torch.randn(E * 2 * ff + 2 * ffs, W) * 0.2
+    dn = torch.randn(W, E * ff + ffs) * 0.2
+    z = torch.randn(T, E)
+    wr = ref_route(z.to(F64), top)
+    ref = torch.zeros(T, W, dtype=F64)
+    for e in range(E + (1 if ffs else 0)):
+        n = ff if e < E else ffs
+        b = gu[e * 2 * ff:e * 2 * ff + 2 * n].to(F64)
+        y = (torch.nn.functional.silu(h.to(F64) @ b[:n].T) * (h.to(F64) @ b[n:].T)) \
+            @ dn[:, e * ff:e * ff + n].to(F64).T
+        ref += y * (wr[:, e:e + 1] if e < E else 1.0)
+    hd, gd, dd = h.to(DEV), gu.to(DEV), dn.to(DEV)
+    wts = M.route_topk(z.to(DEV), top)
+    for fn in (M.moe_dense, M.moe_grouped):
+        torch.testing.assert_close(fn(hd, wts, gd, dd, E, ff, ffs).cpu().to(F64), ref, rtol=1e-4,
+                                   atol=1e-4)
+    torch.testing.assert_close(M.moe(hd, wts, gd, dd, E, top, ff, ffs).cpu().to(F64), ref,
+                               rtol=1e-4, atol=1e-4)
