@@ -5,9 +5,9 @@
 // `sink` adds a key of score 0 that carries no value, i.e. the running softmax starts from
 // (max 0, denominator 1) instead of (-inf, 0).
 //
-// One wave per (row, query head), for prefill chunks and decode rows alike (a row is a row: its
+// Four waves per (row, query head), for prefill chunks and decode rows alike (a row is a row: its
 // position and its segment's block table say which keys it sees, so the result cannot depend on
-// how the step was cut).  Keys are visited 64 at a time: lane l scores key j0 + l -- the dot
+// how the step was cut).  The waves take the 64-key tiles in turn; within a tile lane l scores key j0 + l -- the dot
 // product and the key's sum of squares come from the same 16-byte loads -- then the wave takes
 // the tile's max and sum (online softmax), and for the value pass lane l owns channels l, l + 64,
 // ... of the output and walks the tile's keys (coalesced rows).  Scores, norms and the softmax
@@ -21,35 +21,41 @@ namespace {
 
 constexpr int kMaxD = 256;
 
+constexpr int kRowWaves = 4;   // waves per (row, head): each takes every fourth 64-key tile
+
 template <typename T>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(64 * kRowWaves)
 chunk_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ cache,
                   T* __restrict__ out, const int* __restrict__ tables, int maxb,
                   const int* __restrict__ row_seg, const int* __restrict__ positions, int H, int G,
                   int D, int bs, float scale, float eps, int chunk, int sink) {
-  const int t = blockIdx.x, hd = blockIdx.y, lane = threadIdx.x;
+  const int t = blockIdx.x, hd = blockIdx.y, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int g = hd / (H / G);
   const int pos = positions[t];
   const int* tbl = tables + (long long)row_seg[t] * maxb;
   const int lo = chunk > 0 ? (pos / chunk) * chunk : 0;
   __shared__ float s_q[kMaxD];
-  __shared__ float s_p[64];
-  __shared__ long long s_row[64];
+  __shared__ float s_p[kRowWaves][64];
+  __shared__ long long s_row[kRowWaves][64];
+  __shared__ float s_acc[kRowWaves][kMaxD];
+  __shared__ float s_m[kRowWaves], s_l[kRowWaves];
 
   float ss = 0.f;
   for (int d = lane; d < D; d += 64) {
     const float v = to_f32(q[(long long)t * ldq + hd * D + d]);
-    s_q[d] = v;
+    if (w == 0) s_q[d] = v;
     ss += v * v;
   }
   ss = wave_sum(ss);
   const float qn = scale / sqrtf(ss / D + eps);
   __syncthreads();
 
-  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  // every wave keeps its own running (max, sum, accumulator) over its tiles; wave 0 starts from
+  // the sink, the others from nothing, and the partial results are merged at the end
+  float m = (sink && w == 0) ? 0.f : -INFINITY, l = (sink && w == 0) ? 1.f : 0.f;
   float acc[kMaxD / 64] = {0.f, 0.f, 0.f, 0.f};
   const bool vec = (D % 8) == 0;
-  for (int j0 = lo; j0 <= pos; j0 += 64) {
+  for (int j0 = lo + 64 * w; j0 <= pos; j0 += 64 * kRowWaves) {
     const int j = j0 + lane;
     const bool valid = j <= pos;
     float s = -INFINITY;
@@ -74,33 +80,53 @@ chunk_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ 
       }
       s = dot * qn / sqrtf(k2 / D + eps);
     }
-    const float mn = fmaxf(m, wave_max(s));
+    const float mn = fmaxf(m, wave_max(s));       // finite: the tile's first key is valid
     const float p = valid ? expf(s - mn) : 0.f;
-    const float corr = expf(m - mn);       // m = -inf only before the first tile without a sink
+    const float corr = expf(m - mn);
     l = l * corr + wave_sum(p);
     m = mn;
-    s_p[lane] = p;
-    s_row[lane] = rowoff;
-    __syncthreads();
+    s_p[w][lane] = p;
+    s_row[w][lane] = rowoff;
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     const int nk = min(64, pos - j0 + 1);
 #pragma unroll
     for (int c = 0; c < kMaxD / 64; ++c) acc[c] *= corr;
     for (int jj = 0; jj < nk; ++jj) {
-      const float pj = s_p[jj];
-      const T* kp = cache + s_row[jj];
+      const float pj = s_p[w][jj];
+      const T* kp = cache + s_row[w][jj];
 #pragma unroll
       for (int c = 0; c < kMaxD / 64; ++c) {
         const int d = lane + 64 * c;
         if (d < D) acc[c] += pj * to_f32(kp[d]);
       }
     }
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();
   }
-  const float inv = 1.f / l;
+  if (lane == 0) { s_m[w] = m; s_l[w] = l; }
 #pragma unroll
   for (int c = 0; c < kMaxD / 64; ++c) {
     const int d = lane + 64 * c;
-    if (d < D) out[((long long)t * H + hd) * D + d] = from_f32<T>(acc[c] * inv);
+    if (d < D) s_acc[w][d] = acc[c];
+  }
+  __syncthreads();
+  if (w == 0) {
+    float mt = -INFINITY;
+#pragma unroll
+    for (int x = 0; x < kRowWaves; ++x) mt = fmaxf(mt, s_m[x]);
+    float lt = 0.f, f[kRowWaves];
+#pragma unroll
+    for (int x = 0; x < kRowWaves; ++x) {
+      f[x] = s_m[x] == -INFINITY ? 0.f : expf(s_m[x] - mt);
+      lt += s_l[x] * f[x];
+    }
+    const float inv = 1.f / lt;
+    for (int d = lane; d < D; d += 64) {
+      float o = 0.f;
+#pragma unroll
+      for (int x = 0; x < kRowWaves; ++x) o += s_acc[x][d] * f[x];
+      out[((long long)t * H + hd) * D + d] = from_f32<T>(o * inv);
+    }
   }
 }
 
@@ -148,8 +174,11 @@ __device__ __forceinline__ float sumsq8(uint4 v) {
   return s;
 }
 
+// (register budget: three waves per SIMD up to head size 128 -- 168 VGPRs, no scratch -- two
+// above; left to itself the compiler takes > 300 registers and runs one wave per SIMD, which
+// measured slower than the staging it was meant to speed up)
 template <typename T, int D, int NW>
-__global__ void __launch_bounds__(64 * NW)
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(D <= 128 ? 3 : 2)))
 tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ cache,
                  T* __restrict__ out, const int* __restrict__ tables, int maxb,
                  const int* __restrict__ tiles, const int* __restrict__ cu,
@@ -277,17 +306,20 @@ tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ c
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
     const float mn = fmaxf(m, mloc);
     const float ms = mn == -INFINITY ? 0.f : mn;
-    const float corr = expf(m - ms);
+    // (v_exp_f32: this kernel serves 16-bit dtypes only, the weights are rounded to ~16 bits)
+    const float corr = __expf(m - ms);
     float psum = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { sc[r] = expf(sc[r] - ms); psum += sc[r]; }
+    for (int r = 0; r < 16; ++r) { sc[r] = __expf(sc[r] - ms); psum += sc[r]; }
     psum += __shfl_xor(psum, 32, 64);
     l = l * corr + psum;
     m = mn;
+    if (__any(corr != 1.f)) {              // the running max moved for some query of the wave
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db)
+      for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) O[db][r] *= corr;
+        for (int r = 0; r < 16; ++r) O[db][r] *= corr;
+    }
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2) {
       unsigned ph[4], pl[4];
@@ -382,7 +414,7 @@ hipError_t sm_chunk_attn(int dt, const void* q, long long ldq, const void* cache
   if (T == 0) return hipSuccess;
   if (D < 1 || D > kMaxD || G < 1 || H % G || bs < 1 || chunk < 0) return hipErrorInvalidValue;
   const dim3 grid(T, H);
-#define CALL(TT) chunk_attn_kernel<TT><<<grid, 64, 0, st>>>((const TT*)q, ldq, (const TT*)cache, (TT*)out, tables, maxb, row_seg, positions, H, G, D, bs, scale, eps, chunk, sink)
+#define CALL(TT) chunk_attn_kernel<TT><<<grid, 64 * kRowWaves, 0, st>>>((const TT*)q, ldq, (const TT*)cache, (TT*)out, tables, maxb, row_seg, positions, H, G, D, bs, scale, eps, chunk, sink)
   SM_DISPATCH(dt, CALL)
 #undef CALL
   return hipGetLastError();

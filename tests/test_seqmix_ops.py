@@ -167,7 +167,7 @@ def _scan_inputs(H, D, dtype, seed, n_in):
 
 
 @pytest.mark.parametrize("dev,dtype,pieces", CASES)
-@pytest.mark.parametrize("H,D", [(2, 32), (3, 48), (1, 64), (2, 80)])
+@pytest.mark.parametrize("H,D", [(2, 32), (3, 48), (1, 64), (2, 80), (1, 256)])
 def test_wkv_scan_segments(dev, dtype, pieces, H, D):
     from lumen.ops.recurrent import wkv_scan
 
@@ -194,7 +194,7 @@ def test_wkv_scan_segments(dev, dtype, pieces, H, D):
 
 
 @pytest.mark.parametrize("dev,dtype,pieces", CASES)
-@pytest.mark.parametrize("H,D", [(2, 32), (3, 48), (1, 128)])
+@pytest.mark.parametrize("H,D", [(2, 32), (3, 48), (1, 128), (1, 200)])
 def test_delta_scan_segments(dev, dtype, pieces, H, D):
     from lumen.ops.recurrent import delta_scan
 
