@@ -83,6 +83,40 @@ __global__ void gated_act_kernel(const T* __restrict__ gu, const float* __restri
   }
 }
 
+// eight outputs per thread (16-byte accesses): every block size a multiple of 8, 16-bit dtypes
+template <typename T>
+__global__ void __launch_bounds__(256)
+gated_act_v8(const T* __restrict__ gu, const float* __restrict__ wts, T* __restrict__ out, int Tn,
+             int E, int ff, int ffs) {
+  const int in_w = E * 2 * ff + 2 * ffs, out_w = E * ff + ffs;
+  const int c = 8 * (blockIdx.x * 256 + threadIdx.x);
+  if (c >= out_w) return;
+  int e = -1, goff, uoff;
+  if (c < E * ff) {
+    e = c / ff;
+    goff = e * 2 * ff + (c - e * ff);
+    uoff = goff + ff;
+  } else {
+    goff = E * 2 * ff + (c - E * ff);
+    uoff = goff + ffs;
+  }
+  for (int t = blockIdx.y; t < Tn; t += gridDim.y) {
+    const T* row = gu + (long long)t * in_w;
+    const float w = e >= 0 ? wts[(long long)t * E + e] : 1.f;
+    float g[8], u[8], o[8];
+    if (w == 0.f) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = 0.f;
+    } else {
+      load8<T>(row + goff, g);
+      load8<T>(row + uoff, u);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = silu_f(g[j]) * u[j] * w;
+    }
+    store8<T>(out + (long long)t * out_w + c, o);
+  }
+}
+
 template <typename T>
 __global__ void write_k_kernel(const T* __restrict__ k, long long ld, T* __restrict__ cache,
                                const long long* __restrict__ slots, int Tn, int GD) {
@@ -116,6 +150,14 @@ hipError_t sm_gated_act(int dt, const void* gu, const float* wts, void* out, int
   const long long n = (long long)T * (E * ff + ffs);
   if (n == 0) return hipSuccess;
   if (E > 0 && wts == nullptr) return hipErrorInvalidValue;
+  if (ff % 8 == 0 && ffs % 8 == 0 && (dt == kBF16 || dt == kF16)) {
+    const dim3 grid(((E * ff + ffs) / 8 + 255) / 256, T < 65535 ? T : 65535);
+    if (dt == kBF16)
+      gated_act_v8<bf16><<<grid, 256, 0, st>>>((const bf16*)gu, wts, (bf16*)out, T, E, ff, ffs);
+    else
+      gated_act_v8<fp16><<<grid, 256, 0, st>>>((const fp16*)gu, wts, (fp16*)out, T, E, ff, ffs);
+    return hipGetLastError();
+  }
 #define CALL(TT) gated_act_kernel<TT><<<grid_for(n), 256, 0, st>>>((const TT*)gu, wts, (TT*)out, T, E, ff, ffs)
   SM_DISPATCH(dt, CALL)
 #undef CALL

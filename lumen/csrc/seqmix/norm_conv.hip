@@ -6,9 +6,11 @@
 //   sm_canon_tail    the tail moves on to the segment's last taps - 1 normed rows
 //   sm_token_shift   out[s] = h + (h_prev - h) * mu[s], h_prev the previous row of the sequence
 //   sm_shift_tail    prev[slot] = the segment's last row
-// All are memory-bound element-wise passes: one thread per element, grid-stride, consecutive
-// threads on consecutive channels (coalesced rows); DyT of a neighbouring row is recomputed from
-// x (a tanh) rather than staged, so x is read taps times through L2 and written nowhere.
+// All are memory-bound passes.  When the width is a multiple of 4 a thread owns FOUR consecutive
+// channels (16-byte fp32 / 8-byte 16-bit accesses), rows come from the grid's y dimension (no
+// index division), per-channel constants are loaded once per thread; the convolution walks a
+// strip of rows with the last taps - 1 normed rows in registers, so every tanh is computed once
+// (plus the strip's halo).  Other widths take the one-element-per-thread kernels.
 #include "seqmix.h"
 
 using namespace lumen;
@@ -148,6 +150,127 @@ __global__ void shift_tail_kernel(const T* __restrict__ h, float* __restrict__ p
   }
 }
 
+// ---- four channels per thread ------------------------------------------------------------------
+template <typename TY, typename TH>
+__global__ void __launch_bounds__(256)
+dyt_residual_v4(float* __restrict__ x, const TY* __restrict__ y, const float* __restrict__ pw,
+                const float* __restrict__ pb, const float* __restrict__ pa, TH* __restrict__ h,
+                const float* __restrict__ w2, const float* __restrict__ b2,
+                const float* __restrict__ a2, int T, int W) {
+  const int c = 4 * (blockIdx.x * 256 + threadIdx.x);
+  if (c >= W) return;
+  const float ap = *pa, an = h ? *a2 : 0.f;
+  float w1[4], b1[4], wn[4] = {0, 0, 0, 0}, bn[4] = {0, 0, 0, 0};
+  load4<float>(pw + c, w1);
+  load4<float>(pb + c, b1);
+  if (h) { load4<float>(w2 + c, wn); load4<float>(b2 + c, bn); }
+  for (int t = blockIdx.y; t < T; t += gridDim.y) {
+    const long long i = (long long)t * W + c;
+    float xv[4], yv[4], hv[4];
+    load4<float>(x + i, xv);
+    load4<TY>(y + i, yv);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      xv[j] += dyt_f(yv[j], ap, w1[j], b1[j]);
+      hv[j] = dyt_f(xv[j], an, wn[j], bn[j]);
+    }
+    store4<float>(x + i, xv);
+    if (h) store4<TH>(h + i, hv);
+  }
+}
+
+constexpr int kStrip = 16;   // rows per workgroup of the convolution
+
+template <typename TO, int TAPS>
+__global__ void __launch_bounds__(64)
+dyt_canon_v4(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ b,
+             const float* __restrict__ alpha, const float* __restrict__ cw,
+             const float* __restrict__ tail, TO* __restrict__ out, const int* __restrict__ cu,
+             const int* __restrict__ slot, const int* __restrict__ start,
+             const int* __restrict__ row_seg, int T, int W) {
+  constexpr int K = TAPS - 1;
+  const int c = 4 * (blockIdx.x * 64 + threadIdx.x);
+  if (c >= W) return;
+  const float a = *alpha;
+  float wv[4], bv[4], cwv[4][TAPS];
+  load4<float>(w + c, wv);
+  load4<float>(b + c, bv);
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int q = 0; q < TAPS; ++q) cwv[j][q] = cw[(long long)(c + j) * TAPS + q];
+  float win[K > 0 ? K : 1][4];        // win[d - 1]: the normed row d positions back
+  const int r0 = blockIdx.y * kStrip, r1 = min(T, r0 + kStrip);
+  int cur = -1;
+  for (int t = r0; t < r1; ++t) {
+    const int sg = row_seg[t];
+    const long long i = (long long)t * W + c;
+    if (sg != cur) {                   // strip start or a new segment: rebuild the window
+      cur = sg;
+      const int local = t - cu[sg], p0 = start[sg];
+#pragma unroll
+      for (int d = 1; d <= K; ++d) {
+        const int src = local - d;
+        float hv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (src >= 0) {
+          load4<float>(x + i - (long long)d * W, hv);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) hv[j] = dyt_f(hv[j], a, wv[j], bv[j]);
+        } else if (p0 + src >= 0) {
+          load4<float>(tail + ((long long)slot[sg] * K + (K + src)) * W + c, hv);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) win[d - 1][j] = hv[j];
+      }
+    }
+    float hc[4], o[4];
+    load4<float>(x + i, hc);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      hc[j] = dyt_f(hc[j], a, wv[j], bv[j]);
+      float acc = cwv[j][K] * hc[j];
+#pragma unroll
+      for (int d = 1; d <= K; ++d) acc += cwv[j][K - d] * win[d - 1][j];
+      o[j] = hc[j] + acc;
+    }
+    store4<TO>(out + i, o);
+#pragma unroll
+    for (int d = K; d >= 2; --d)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) win[d - 1][j] = win[d - 2][j];
+    if (K > 0) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) win[0][j] = hc[j];
+    }
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+token_shift_v4(const T* __restrict__ h, const float* __restrict__ mu, const float* __restrict__ prev,
+               T* __restrict__ out, const int* __restrict__ cu, const int* __restrict__ slot,
+               const int* __restrict__ start, const int* __restrict__ row_seg, int Tn, int W,
+               int nmix) {
+  const int c = 4 * (blockIdx.x * 256 + threadIdx.x);
+  if (c >= W) return;
+  const long long n = (long long)Tn * W;
+  for (int t = blockIdx.y; t < Tn; t += gridDim.y) {
+    const int sg = row_seg[t];
+    const long long i = (long long)t * W + c;
+    float hv[4], pv[4] = {0.f, 0.f, 0.f, 0.f};
+    load4<T>(h + i, hv);
+    if (t > cu[sg]) load4<T>(h + i - W, pv);
+    else if (start[sg] > 0) load4<float>(prev + (long long)slot[sg] * W + c, pv);
+    for (int s = 0; s < nmix; ++s) {
+      float m4[4], o[4];
+      load4<float>(mu + (long long)s * W + c, m4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = hv[j] + (pv[j] - hv[j]) * m4[j];
+      store4<T>(out + (long long)s * n + i, o);
+    }
+  }
+}
+
 inline int grid_for(long long n, int block = 256) {
   long long g = (n + block - 1) / block;
   return (int)(g < 1 ? 1 : (g > 65536 ? 65536 : g));
@@ -174,6 +297,13 @@ hipError_t sm_dyt_residual(int dt_y, int dt_h, float* x, const void* y, const fl
   const long long n = (long long)T * W;
   if (n == 0) return hipSuccess;
   if (h && dt_h != dt_y) return hipErrorInvalidValue;
+  if (W % 4 == 0) {
+    const dim3 grid((W / 4 + 255) / 256, T < 65535 ? T : 65535);
+#define CALL(TT) dyt_residual_v4<TT, TT><<<grid, 256, 0, st>>>(x, (const TT*)y, pw, pb, pa, (TT*)h, w2, b2, a2, T, W)
+    SM_DISPATCH(dt_y, CALL)
+#undef CALL
+    return hipGetLastError();
+  }
 #define CALL(TT) dyt_residual_kernel<TT, TT><<<grid_for(n), 256, 0, st>>>(x, (const TT*)y, pw, pb, pa, (TT*)h, w2, b2, a2, n, W)
   SM_DISPATCH(dt_y, CALL)
 #undef CALL
@@ -186,6 +316,20 @@ hipError_t sm_dyt_canon(int dt, const float* x, const float* w, const float* b, 
                         int taps, hipStream_t st) {
   if ((long long)T * W == 0) return hipSuccess;
   if (taps < 1 || taps > kMaxTaps) return hipErrorInvalidValue;
+  if (W % 4 == 0 && taps <= 8) {
+    const dim3 grid((W / 4 + 63) / 64, (T + kStrip - 1) / kStrip);
+#define GO(TT, TP) dyt_canon_v4<TT, TP><<<grid, 64, 0, st>>>(x, w, b, alpha, cw, tail, (TT*)out, cu, slot, start, row_seg, T, W)
+#define CALL(TT)                                                                     \
+    switch (taps) {                                                                  \
+      case 1: GO(TT, 1); break; case 2: GO(TT, 2); break; case 3: GO(TT, 3); break;  \
+      case 4: GO(TT, 4); break; case 5: GO(TT, 5); break; case 6: GO(TT, 6); break;  \
+      case 7: GO(TT, 7); break; default: GO(TT, 8); break;                           \
+    }
+    SM_DISPATCH(dt, CALL)
+#undef CALL
+#undef GO
+    return hipGetLastError();
+  }
 #define CALL(TT) dyt_canon_kernel<TT><<<grid_for((long long)T * W), 256, 0, st>>>(x, w, b, alpha, cw, tail, (TT*)out, cu, slot, start, row_seg, T, W, taps)
   SM_DISPATCH(dt, CALL)
 #undef CALL
@@ -206,6 +350,13 @@ hipError_t sm_token_shift(int dt, const void* h, const float* mu, const float* p
                           const int* cu, const int* slot, const int* start, const int* row_seg,
                           int T, int W, int nmix, hipStream_t st) {
   if ((long long)T * W == 0) return hipSuccess;
+  if (W % 4 == 0) {
+    const dim3 grid((W / 4 + 255) / 256, T < 65535 ? T : 65535);
+#define CALL(TT) token_shift_v4<TT><<<grid, 256, 0, st>>>((const TT*)h, mu, prev, (TT*)out, cu, slot, start, row_seg, T, W, nmix)
+    SM_DISPATCH(dt, CALL)
+#undef CALL
+    return hipGetLastError();
+  }
 #define CALL(TT) token_shift_kernel<TT><<<grid_for((long long)T * W), 256, 0, st>>>((const TT*)h, mu, prev, (TT*)out, cu, slot, start, row_seg, T, W, nmix)
   SM_DISPATCH(dt, CALL)
 #undef CALL

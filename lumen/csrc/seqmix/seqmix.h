@@ -13,6 +13,24 @@ __device__ __forceinline__ float dyt_f(float x, float alpha, float w, float b) {
   return tanhf(alpha * x) * w + b;
 }
 
+// four consecutive elements as one vector access (16 bytes of fp32, 8 bytes of a 16-bit type)
+template <typename T> __device__ __forceinline__ void load4(const T* __restrict__ p, float (&o)[4]) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(p);
+  const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = to_f32(e[j]);
+}
+template <> __device__ __forceinline__ void load4<float>(const float* __restrict__ p, float (&o)[4]) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+}
+template <typename T> __device__ __forceinline__ void store4(T* __restrict__ p, const float (&v)[4]) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pk2<T>(v[0], v[1]), pk2<T>(v[2], v[3]));
+}
+template <> __device__ __forceinline__ void store4<float>(float* __restrict__ p, const float (&v)[4]) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+
 }  // namespace lumen
 
 // run `CALL(T)` with T = float / fp16 / bf16 for dtype code `dt`

@@ -96,12 +96,12 @@ DEVS = ["cpu", pytest.param("cuda", marks=GPU)]
 
 
 @pytest.mark.parametrize("dev,dtype,pieces", CASES)
-@pytest.mark.parametrize("taps", [1, 2, 4])
-def test_dyt_canon_segments(dev, dtype, pieces, taps):
+@pytest.mark.parametrize("taps,W", [(1, 96), (2, 96), (4, 96), (3, 50), (10, 24)])
+def test_dyt_canon_segments(dev, dtype, pieces, taps, W):
+    """(Widths that are / are not a multiple of 4 and more than 8 taps take different kernels.)"""
     from lumen.ops.conv import dyt_canon
 
     torch.manual_seed(taps)
-    W = 96
     norm = (torch.randn(W) * 0.2 + 1, torch.randn(W) * 0.1, torch.tensor(0.7))
     cw = torch.randn(W, taps) * 0.4
     xs = [torch.randn(n, W) for n in LENGTHS]
@@ -118,11 +118,12 @@ def test_dyt_canon_segments(dev, dtype, pieces, taps):
 
 @pytest.mark.parametrize("dev,dtype", [("cpu", torch.float32)] + [
     pytest.param("cuda", d, marks=GPU) for d in DTYPES])
-def test_dyt_and_residual(dev, dtype):
+@pytest.mark.parametrize("W", [80, 42])
+def test_dyt_and_residual(dev, dtype, W):
     from lumen.ops.norm import dyt, dyt_residual
 
     torch.manual_seed(0)
-    T, W = 33, 80
+    T = 33
     n1 = (torch.randn(W) + 1, torch.randn(W) * 0.1, torch.tensor(0.4))
     n2 = (torch.randn(W) + 1, torch.randn(W) * 0.1, torch.tensor(1.3))
     x, y = torch.randn(T, W), torch.randn(T, W).to(dtype)
@@ -140,11 +141,11 @@ def test_dyt_and_residual(dev, dtype):
 
 
 @pytest.mark.parametrize("dev,dtype,pieces", CASES)
-def test_token_shift_segments(dev, dtype, pieces):
+@pytest.mark.parametrize("W", [72, 30])
+def test_token_shift_segments(dev, dtype, pieces, W):
     from lumen.ops.recurrent import token_shift
 
     torch.manual_seed(2)
-    W = 72
     mu = torch.rand(5, W)
     hs = [torch.randn(n, W).to(dtype) for n in LENGTHS]
     ref = [ref_token_shift(h.to(F64), mu.to(F64)) for h in hs]
@@ -321,7 +322,7 @@ def test_route_topk(dev, E, top):
 
 @pytest.mark.parametrize("dev,dtype", [("cpu", torch.float32)] + [
     pytest.param("cuda", d, marks=GPU) for d in DTYPES])
-@pytest.mark.parametrize("E,ff,ffs", [(0, 0, 96), (5, 24, 40), (3, 16, 0)])
+@pytest.mark.parametrize("E,ff,ffs", [(0, 0, 96), (5, 24, 40), (3, 16, 0), (4, 12, 20)])
 def test_gated_act(dev, dtype, E, ff, ffs):
     from lumen.ops.moe import gated_act
 
