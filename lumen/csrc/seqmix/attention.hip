@@ -54,7 +54,10 @@ chunk_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ 
   // the sink, the others from nothing, and the partial results are merged at the end
   float m = (sink && w == 0) ? 0.f : -INFINITY, l = (sink && w == 0) ? 1.f : 0.f;
   float acc[kMaxD / 64] = {0.f, 0.f, 0.f, 0.f};
+  float acc8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const bool vec = (D % 8) == 0;
+  const int lpk = vec ? D / 8 : 64, kpi = 64 / lpk;   // lanes per key row, keys per step
+  const int grp = lane / lpk, part = lane % lpk;
   for (int j0 = lo + 64 * w; j0 <= pos; j0 += 64 * kRowWaves) {
     const int j = j0 + lane;
     const bool valid = j <= pos;
@@ -90,25 +93,55 @@ chunk_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ 
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     const int nk = min(64, pos - j0 + 1);
+    if (vec) {
+      // value pass, 16 bytes per lane: lpk = D / 8 lanes cover one key row, 64 / lpk keys per
+      // step; a lane accumulates its 8 channels over the keys of its group, the groups are
+      // summed once at the end
 #pragma unroll
-    for (int c = 0; c < kMaxD / 64; ++c) acc[c] *= corr;
-    for (int jj = 0; jj < nk; ++jj) {
-      const float pj = s_p[w][jj];
-      const T* kp = cache + s_row[w][jj];
+      for (int e = 0; e < 8; ++e) acc8[e] *= corr;
+      if (grp < kpi) {
+        for (int jj = grp; jj < nk; jj += kpi) {
+          const float pj = s_p[w][jj];
+          float kv[8];
+          load8<T>(cache + s_row[w][jj] + 8 * part, kv);
 #pragma unroll
-      for (int c = 0; c < kMaxD / 64; ++c) {
-        const int d = lane + 64 * c;
-        if (d < D) acc[c] += pj * to_f32(kp[d]);
+          for (int e = 0; e < 8; ++e) acc8[e] += pj * kv[e];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < kMaxD / 64; ++c) acc[c] *= corr;
+      for (int jj = 0; jj < nk; ++jj) {
+        const float pj = s_p[w][jj];
+        const T* kp = cache + s_row[w][jj];
+#pragma unroll
+        for (int c = 0; c < kMaxD / 64; ++c) {
+          const int d = lane + 64 * c;
+          if (d < D) acc[c] += pj * to_f32(kp[d]);
+        }
       }
     }
     __builtin_amdgcn_wave_barrier();
   }
-  if (lane == 0) { s_m[w] = m; s_l[w] = l; }
+  if (vec) {
+    // sum the key groups of this wave: every group adds its channels into s_acc[w] in turn
+    for (int d = lane; d < D; d += 64) s_acc[w][d] = 0.f;
+    for (int gq = 0; gq < kpi; ++gq) {
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      if (grp == gq) {
 #pragma unroll
-  for (int c = 0; c < kMaxD / 64; ++c) {
-    const int d = lane + 64 * c;
-    if (d < D) s_acc[w][d] = acc[c];
+        for (int e = 0; e < 8; ++e) s_acc[w][8 * part + e] += acc8[e];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < kMaxD / 64; ++c) {
+      const int d = lane + 64 * c;
+      if (d < D) s_acc[w][d] = acc[c];
+    }
   }
+  if (lane == 0) { s_m[w] = m; s_l[w] = l; }
   __syncthreads();
   if (w == 0) {
     float mt = -INFINITY;
@@ -187,6 +220,8 @@ tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ c
   constexpr int QT = 32 * NW, LK = D + 8, LT = 40, NV = D / 8;
   __shared__ __align__(16) T s_k[32 * LK];    // key tile, row-major
   __shared__ __align__(16) T s_t[D * LT];     // key tile, transposed [d][key]
+  __shared__ float s_kn[32];                  // 1 / rms of the tile's keys (power-of-two D / 8)
+  constexpr bool kStagedNorm = (NV & (NV - 1)) == 0 && NV <= 64;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c = lane & 31, hi = lane >> 5;
   const int hd = blockIdx.y, g = hd / (H / G);
   const int sg = tiles[2 * blockIdx.x], row0 = tiles[2 * blockIdx.x + 1];
@@ -255,6 +290,15 @@ tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ c
 #pragma unroll
         for (int x = 0; x < 4; ++x)
           *reinterpret_cast<uint4*>(&s_k[(4 * kq + x) * LK + 8 * part]) = pre[it][x];
+        if (kStagedNorm) {   // the NV lanes of a key quad are adjacent: sum their partial squares
+#pragma unroll
+          for (int x = 0; x < 4; ++x) {
+            float k2 = sumsq8<T>(pre[it][x]);
+#pragma unroll
+            for (int o = 1; o < NV; o <<= 1) k2 += __shfl_xor(k2, o, 64);
+            if (part == 0) s_kn[4 * kq + x] = 1.f / sqrtf(k2 / D + eps);
+          }
+        }
         const unsigned w0[4] = {pre[it][0].x, pre[it][0].y, pre[it][0].z, pre[it][0].w};
         const unsigned w1[4] = {pre[it][1].x, pre[it][1].y, pre[it][1].z, pre[it][1].w};
         const unsigned w2[4] = {pre[it][2].x, pre[it][2].y, pre[it][2].z, pre[it][2].w};
@@ -286,20 +330,25 @@ tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ c
 #pragma unroll
     for (int kk = 0; kk < D / 16; ++kk) {
       const uint4 a = *reinterpret_cast<const uint4*>(&s_k[c * LK + 16 * kk + 8 * hi]);
-      k2 += sumsq8<T>(a);
+      if (!kStagedNorm) k2 += sumsq8<T>(a);
       acc = Mma32<T>::run(a, qreg[kk], acc);
     }
-    k2 += __shfl_xor(k2, 32, 64);
-    const float kn = 1.f / sqrtf(k2 / D + eps);          // of key k0 + c
-
+    float kn = 0.f;                                      // of key k0 + c (other head sizes)
+    if (!kStagedNorm) {
+      k2 += __shfl_xor(k2, 32, 64);
+      kn = 1.f / sqrtf(k2 / D + eps);
+    }
+    // a tile every query of the wave sees whole needs no mask
+    const bool whole = k0 >= (chunk > 0 ? (wpos_max / chunk) * chunk : 0) && k0 + 31 <= wpos_min &&
+                       32 * w + 31 < nrows;
     float sc[16];
     float mloc = -INFINITY;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int keyr = 8 * (r >> 2) + 4 * hi + (r & 3);
       const int j = k0 + keyr;
-      const float knr = __shfl(kn, keyr, 64);
-      const bool ok = j >= lo && j <= pos;
+      const float knr = kStagedNorm ? s_kn[keyr] : __shfl(kn, keyr, 64);
+      const bool ok = whole || (j >= lo && j <= pos);
       sc[r] = ok ? acc[r] * qn * knr : -INFINITY;
       mloc = fmaxf(mloc, sc[r]);
     }
@@ -362,12 +411,17 @@ template <typename T>
 hipError_t launch_tiles(const void* q, long long ldq, const void* cache, void* out,
                         const int* tables, int maxb, const int* tiles, int ntiles, const int* cu,
                         const int* start, int H, int G, int D, int bs, float scale, float eps,
-                        int chunk, int sink, hipStream_t st) {
+                        int chunk, int sink, int tile_rows, hipStream_t st) {
   const dim3 grid(ntiles, H);
-#define GO(DD)                                                                                  \
-  tile_attn_kernel<T, DD, 2><<<grid, 128, 0, st>>>((const T*)q, ldq, (const T*)cache, (T*)out,  \
-                                                   tables, maxb, tiles, cu, start, H, G, bs,    \
-                                                   scale, eps, chunk, sink)
+#define GO(DD)                                                                                   \
+  if (tile_rows == 128)                                                                          \
+    tile_attn_kernel<T, DD, 4><<<grid, 256, 0, st>>>((const T*)q, ldq, (const T*)cache, (T*)out, \
+                                                     tables, maxb, tiles, cu, start, H, G, bs,   \
+                                                     scale, eps, chunk, sink);                   \
+  else                                                                                           \
+    tile_attn_kernel<T, DD, 2><<<grid, 128, 0, st>>>((const T*)q, ldq, (const T*)cache, (T*)out, \
+                                                     tables, maxb, tiles, cu, start, H, G, bs,   \
+                                                     scale, eps, chunk, sink)
   switch (D) {
     case 32: GO(32); break;
     case 64: GO(64); break;
@@ -391,19 +445,22 @@ int sm_chunk_attn_tiles_ok(int dt, int D) {
          (D == 32 || D == 64 || D == 96 || D == 128 || D == 192 || D == 256);
 }
 
-// tiles: [ntiles, 2] int32 (segment, first row); every tile covers up to 64 rows of its segment
+// tiles: [ntiles, 2] int32 (segment, first row); every tile covers up to tile_rows (64 or 128)
+// rows of its segment
 hipError_t sm_chunk_attn_tiles(int dt, const void* q, long long ldq, const void* cache, void* out,
                                const int* tables, int maxb, const int* tiles, int ntiles,
                                const int* cu, const int* start, int H, int G, int D, int bs,
-                               float scale, float eps, int chunk, int sink, hipStream_t st) {
+                               float scale, float eps, int chunk, int sink, int tile_rows,
+                               hipStream_t st) {
   if (ntiles == 0) return hipSuccess;
   if (G < 1 || H % G || bs < 1 || chunk < 0 || (ldq % 8) != 0) return hipErrorInvalidValue;
+  if (tile_rows != 64 && tile_rows != 128) return hipErrorInvalidValue;
   if (dt == kBF16)
     return launch_tiles<bf16>(q, ldq, cache, out, tables, maxb, tiles, ntiles, cu, start, H, G, D,
-                              bs, scale, eps, chunk, sink, st);
+                              bs, scale, eps, chunk, sink, tile_rows, st);
   if (dt == kF16)
     return launch_tiles<fp16>(q, ldq, cache, out, tables, maxb, tiles, ntiles, cu, start, H, G, D,
-                              bs, scale, eps, chunk, sink, st);
+                              bs, scale, eps, chunk, sink, tile_rows, st);
   return hipErrorInvalidValue;
 }
 

@@ -30,7 +30,7 @@ SIGNATURES = {
     "sm_gdelta": "iplplplplplplppppplpppiiifff",
     "sm_write_k": "iplppii",
     "sm_chunk_attn": "iplpppippiiiiiffii",
-    "sm_chunk_attn_tiles": "iplpppipippiiiiffii",
+    "sm_chunk_attn_tiles": "iplpppipippiiiiffiii",
     "sm_route_topk": "ppiii",
     "sm_gated_act": "ipppiiii",
 }

@@ -574,7 +574,7 @@ def chunk_sink_attention(q: torch.Tensor, cache: torch.Tensor, seg, H: int, G: i
         Tp = seg.tile_rows
         call("sm_chunk_attn_tiles", DT[q.dtype], q, q.stride(0), cache, out, seg.tables, maxb,
              seg.q_tiles, seg.q_tiles.shape[0], seg.cu, seg.start, H, G, D, bs, scale, eps, chunk,
-             int(sink))
+             int(sink), seg.tile_size)
     if T > Tp:
         call("sm_chunk_attn", DT[q.dtype], q[Tp:], q.stride(0), cache, out[Tp:], seg.tables, maxb,
              seg.row_seg[Tp:], seg.positions[Tp:], T - Tp, H, G, D, bs, scale, eps, chunk,

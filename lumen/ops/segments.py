@@ -26,6 +26,7 @@ class SegBatch:
     # (the prefill chunks; decode rows follow and take the row kernel).  None: row kernel only.
     q_tiles: Optional[torch.Tensor] = None
     tile_rows: int = 0
+    tile_size: int = 64       # rows per tile of q_tiles (TILE_ROWS when they were cut)
 
     @property
     def S(self) -> int:
@@ -36,13 +37,18 @@ class SegBatch:
         return self.row_seg.shape[0]
 
 
-TILE_ROWS = 64
+import os
+
+# rows per prefill attention tile: 128 (four waves per workgroup share a staged key tile; 167 vs
+# 197 us per 4096 x 32-head x 128 call at 512-token prompts) or 64 (two)
+TILE_ROWS = 64 if os.environ.get("LUMEN_ATTN_TILE_ROWS", "128") == "64" else 128
 
 
-def tile_list(cu, n_segments: int):
+def tile_list(cu, n_segments: int, rows: int = 0):
     """[(segment, first row)] covering the first ``n_segments`` segments of row offsets ``cu``
-    (host ints) in tiles of TILE_ROWS rows."""
-    return [(s, r) for s in range(n_segments) for r in range(int(cu[s]), int(cu[s + 1]), TILE_ROWS)]
+    (host ints) in tiles of ``rows`` (default TILE_ROWS) rows."""
+    rows = rows or TILE_ROWS
+    return [(s, r) for s in range(n_segments) for r in range(int(cu[s]), int(cu[s + 1]), rows)]
 
 
 def whole_sequences(lengths, device, slots=None, block_size: int = 16) -> SegBatch:
@@ -66,4 +72,4 @@ def whole_sequences(lengths, device, slots=None, block_size: int = 16) -> SegBat
     return SegBatch(torch.tensor(cu, **i32),
                     torch.tensor(list(slots) if slots is not None else list(range(S)), **i32),
                     torch.zeros(S, **i32), row_seg, pos, tables, torch.cat(cache_slots),
-                    torch.tensor(tile_list(cu, S), **i32).view(-1, 2), cu[-1])
+                    torch.tensor(tile_list(cu, S), **i32).view(-1, 2), cu[-1], TILE_ROWS)

@@ -475,14 +475,14 @@ class LLMEngine:
             inp.lora_ids = dev[o:o + T].int()
             o += T
         if self.hybrid:
-            from ..ops.segments import SegBatch
+            from ..ops.segments import TILE_ROWS, SegBatch
 
             g = dev[o:o + seg_n].int()
             t0 = 3 * S + 1 + T + S * maxb
             inp.seg = SegBatch(g[:S + 1], g[S + 1:2 * S + 1], g[2 * S + 1:3 * S + 1],
                                g[3 * S + 1:3 * S + 1 + T], inp.positions,
                                g[3 * S + 1 + T:t0].view(S, maxb), inp.slots,
-                               g[t0:].view(-1, 2) if Tp else None, Tp)
+                               g[t0:].view(-1, 2) if Tp else None, Tp, TILE_ROWS)
         return inp
 
     def _to_device(self, host: "np.ndarray") -> torch.Tensor:

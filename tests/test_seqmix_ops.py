@@ -48,7 +48,7 @@ def cut_steps(lengths, pieces, seed):
             yield step
 
 
-def seg_of(step, slots, tables=None, bs=16, tiled=False):
+def seg_of(step, slots, tables=None, bs=16, tiled=False, tile_size=64):
     from lumen.ops.segments import SegBatch, tile_list
 
     i32 = dict(dtype=torch.int32, device=DEV)
@@ -68,8 +68,8 @@ def seg_of(step, slots, tables=None, bs=16, tiled=False):
                   torch.tensor(pos, **i32), tb,
                   torch.tensor(cs, dtype=torch.long, device=DEV) if tables is not None else None)
     if tiled:       # every segment through the matrix-core tiles (where the op has them)
-        sb.q_tiles = torch.tensor(tile_list(cu, len(step)), **i32).view(-1, 2)
-        sb.tile_rows = cu[-1]
+        sb.q_tiles = torch.tensor(tile_list(cu, len(step), tile_size), **i32).view(-1, 2)
+        sb.tile_rows, sb.tile_size = cu[-1], tile_size
     return sb
 
 
@@ -404,10 +404,11 @@ def test_far_token_reaches_through_the_state(dev, kind, pieces):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("pieces", [[1000], [64, 1, 70, 2, 33]])
+@pytest.mark.parametrize("tile_size", [64, 128])
 @pytest.mark.parametrize("H,G,D,chunk,bs", [(4, 2, 128, 48, 16), (2, 1, 96, 100, 16),
                                              (3, 3, 32, 0, 8), (2, 2, 64, 5, 16),
                                              (1, 1, 256, 64, 16), (2, 1, 192, 31, 4)])
-def test_tile_attention_matches_oracle(dtype, pieces, H, G, D, chunk, bs):
+def test_tile_attention_matches_oracle(dtype, pieces, tile_size, H, G, D, chunk, bs):
     """The matrix-core prefill kernel: several 64-row tiles per segment, chunks that start inside
     a tile, span tiles or are smaller than a key tile, segments that start mid-sequence; and the
     row kernel on the same rows gives the same result to rounding."""
@@ -431,7 +432,7 @@ def test_tile_attention_matches_oracle(dtype, pieces, H, G, D, chunk, bs):
     got = [torch.zeros(n, H * D, dtype=F64) for n in lengths]
     rows = [torch.zeros(n, H * D, dtype=F64) for n in lengths]
     for step in cut_steps(lengths, pieces, 6):
-        sg = seg_of(step, slots, tables, bs, tiled=True)
+        sg = seg_of(step, slots, tables, bs, tiled=True, tile_size=tile_size)
         write_key_cache(gather(step, ks).to(DEV), cache, sg.cache_slots)
         qd = gather(step, qs).to(DEV)
         scatter(step, chunk_sink_attention(qd, cache, sg, H, G, D, scale, chunk, eps), got)
