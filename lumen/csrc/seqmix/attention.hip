@@ -198,12 +198,28 @@ template <> struct Mma32<fp16> {
   }
 };
 
+// the two halves of a packed 16-bit pair as fp32 (bf16: a shift and a mask)
+template <typename T> __device__ __forceinline__ void unpack2(unsigned v, float& a, float& b);
+template <> __device__ __forceinline__ void unpack2<bf16>(unsigned v, float& a, float& b) {
+  a = __uint_as_float(v << 16);
+  b = __uint_as_float(v & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void unpack2<fp16>(unsigned v, float& a, float& b) {
+  const lumen_f16x2 h = __builtin_bit_cast(lumen_f16x2, v);
+  a = static_cast<float>(h[0]);
+  b = static_cast<float>(h[1]);
+}
+
 template <typename T>
 __device__ __forceinline__ float sumsq8(uint4 v) {
-  const T* e = reinterpret_cast<const T*>(&v);
+  const unsigned w[4] = {v.x, v.y, v.z, v.w};
   float s = 0.f;
 #pragma unroll
-  for (int x = 0; x < 8; ++x) { const float f = to_f32(e[x]); s += f * f; }
+  for (int x = 0; x < 4; ++x) {
+    float a, b;
+    unpack2<T>(w[x], a, b);
+    s += a * a + b * b;
+  }
   return s;
 }
 
@@ -221,10 +237,14 @@ tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ c
   __shared__ __align__(16) T s_k[32 * LK];    // key tile, row-major
   __shared__ __align__(16) T s_t[D * LT];     // key tile, transposed [d][key]
   __shared__ float s_kn[32];                  // 1 / rms of the tile's keys (power-of-two D / 8)
+  constexpr int kTbl = 512;                   // block-table entries of the visible keys, in LDS
+  __shared__ int s_tbl[kTbl];
   constexpr bool kStagedNorm = (NV & (NV - 1)) == 0 && NV <= 64;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c = lane & 31, hi = lane >> 5;
   const int hd = blockIdx.y, g = hd / (H / G);
-  const int sg = tiles[2 * blockIdx.x], row0 = tiles[2 * blockIdx.x + 1];
+  // tiles are listed in row order, so later tiles see more keys: issue them first
+  const int tix = gridDim.x - 1 - blockIdx.x;
+  const int sg = tiles[2 * tix], row0 = tiles[2 * tix + 1];
   const int seg_r0 = cu[sg], p0 = start[sg];
   const int nrows = min(QT, cu[sg + 1] - row0);
   const int* tbl = tables + (long long)sg * maxb;
@@ -250,6 +270,13 @@ tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ c
   const int wpos_min = pos_first + 32 * w, wpos_max = min(kend, wpos_min + 31);
   const int wlo_min = chunk > 0 ? (wpos_min / chunk) * chunk : 0;
 
+  // the block ids of the keys this tile can see, so that a key's address never waits for a
+  // table load (entries beyond kTbl, i.e. very long chunks, are read from global memory)
+  const int b_first = kbeg / bs, b_count = kend / bs - b_first + 1;
+  for (int i = tid; i < min(b_count, kTbl); i += 64 * NW) s_tbl[i] = tbl[b_first + i];
+  const int bshift = (bs & (bs - 1)) == 0 ? __ffs(bs) - 1 : -1;
+  __syncthreads();
+
   float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
   f32x16 O[D / 32];
 #pragma unroll
@@ -274,7 +301,10 @@ tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ c
           const int j = k0 + 4 * kq + x;
           pre[it][x] = make_uint4(0, 0, 0, 0);
           if (j <= kend) {
-            const long long off = (((long long)tbl[j / bs] * bs + j % bs) * G + g) * D;
+            const int jb = bshift >= 0 ? j >> bshift : j / bs, jo = j - jb * bs;
+            const int bi = jb - b_first;
+            const int blk = bi < kTbl ? s_tbl[bi] : tbl[jb];
+            const long long off = (((long long)blk * bs + jo) * G + g) * D;
             pre[it][x] = *reinterpret_cast<const uint4*>(cache + off + 8 * part);
           }
         }
@@ -305,7 +335,9 @@ tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ c
         const unsigned w3[4] = {pre[it][3].x, pre[it][3].y, pre[it][3].z, pre[it][3].w};
 #pragma unroll
         for (int mm = 0; mm < 4; ++mm) {     // word mm holds channels 2mm (low half), 2mm + 1
-          T* t0 = &s_t[(8 * part + 2 * mm) * LT + 4 * kq];
+          // the key quads of a row are permuted by the row's group of 8 (all rows a lane
+          // writes share it): lanes that differ in `part` land in different banks
+          T* t0 = &s_t[(8 * part + 2 * mm) * LT + 4 * (kq ^ (part & 7))];
           *reinterpret_cast<uint2*>(t0) = make_uint2((w0[mm] & 0xffffu) | (w1[mm] << 16),
                                                      (w2[mm] & 0xffffu) | (w3[mm] << 16));
           *reinterpret_cast<uint2*>(t0 + LT) = make_uint2(
@@ -346,12 +378,18 @@ tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ c
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int keyr = 8 * (r >> 2) + 4 * hi + (r & 3);
-      const int j = k0 + keyr;
       const float knr = kStagedNorm ? s_kn[keyr] : __shfl(kn, keyr, 64);
-      const bool ok = whole || (j >= lo && j <= pos);
-      sc[r] = ok ? acc[r] * qn * knr : -INFINITY;
-      mloc = fmaxf(mloc, sc[r]);
+      sc[r] = acc[r] * qn * knr;
     }
+    if (!whole) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int j = k0 + 8 * (r >> 2) + 4 * hi + (r & 3);
+        sc[r] = (j >= lo && j <= pos) ? sc[r] : -INFINITY;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, sc[r]);
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
     const float mn = fmaxf(m, mloc);
     const float ms = mn == -INFINITY ? 0.f : mn;
@@ -375,17 +413,19 @@ tile_attn_kernel(const T* __restrict__ q, long long ldq, const T* __restrict__ c
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
         const float a0 = sc[8 * s2 + 2 * x], a1 = sc[8 * s2 + 2 * x + 1];
-        const float h0 = to_f32(from_f32<T>(a0)), h1 = to_f32(from_f32<T>(a1));
-        ph[x] = pk2<T>(a0, a1);
+        ph[x] = pk2<T>(a0, a1);                      // one packed conversion
+        float h0, h1;
+        unpack2<T>(ph[x], h0, h1);
         pl[x] = pk2<T>(a0 - h0, a1 - h1);
       }
       const uint4 bh = make_uint4(ph[0], ph[1], ph[2], ph[3]);
       const uint4 bl = make_uint4(pl[0], pl[1], pl[2], pl[3]);
 #pragma unroll
       for (int db = 0; db < D / 32; ++db) {
-        const T* tp = &s_t[(32 * db + c) * LT + 16 * s2 + 4 * hi];
-        const uint2 a0 = *reinterpret_cast<const uint2*>(tp);
-        const uint2 a1 = *reinterpret_cast<const uint2*>(tp + 8);
+        const int row = 32 * db + c, sw = (row >> 3) & 7;     // undo the store's permutation
+        const T* tp = &s_t[row * LT];
+        const uint2 a0 = *reinterpret_cast<const uint2*>(tp + 4 * ((4 * s2 + hi) ^ sw));
+        const uint2 a1 = *reinterpret_cast<const uint2*>(tp + 4 * ((4 * s2 + 2 + hi) ^ sw));
         const uint4 a = make_uint4(a0.x, a0.y, a1.x, a1.y);
         O[db] = Mma32<T>::run(a, bh, O[db]);
         O[db] = Mma32<T>::run(a, bl, O[db]);
