@@ -110,13 +110,16 @@ def validate(cfg: ModelConfig) -> None:
                 raise ValueError(f"layer {i}: the values are the keys, so vdim must equal dim")
             if int(m["mask"]["size"]) < 1:
                 raise ValueError(f"layer {i}: mask.size must be >= 1")
+            if m["dim"] > 256:
+                raise ValueError(f"layer {i}: attention head size {m['dim']} > 256 is not "
+                                 "supported")
         elif m["dim"] > 256:
             raise ValueError(f"layer {i}: recurrent head size {m['dim']} > 256 is not supported")
         f = L.get("mlp")
         if f and f["kind"] == "moe" and not 1 <= f["router"]["top"] <= f["router"]["experts"]:
             raise ValueError(f"layer {i}: top must be in [1, experts]")
-    if cfg.canon_taps < 1:
-        raise ValueError("canon.taps must be >= 1")
+    if not 1 <= cfg.canon_taps <= 16:
+        raise ValueError(f"canon.taps must be in [1, 16], got {cfg.canon_taps}")
 
 
 def _key(name: str) -> str:

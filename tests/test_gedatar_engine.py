@@ -306,6 +306,45 @@ def test_checkpoint_roundtrip_and_strict_names(tmp_path):
         build_model(d, dtype=torch.bfloat16, device="cpu")
 
 
+def test_trace_run_command_line(tmp_path):
+    """bin/trace_run as a user runs it: a checkpoint directory, JSON steps on stdin, one logits
+    file per step that wants any, `done <step>` after every step, exit code 0 at end of input."""
+    import json
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    from lumen.models.loading import save_hf_weights
+
+    m = make("odd", "cpu", dtype=torch.bfloat16)
+    d = str(tmp_path / "ckpt")
+    out = str(tmp_path / "out")
+    save_hf_weights(m, d)
+    a, b = tokens(m, 21, 70), tokens(m, 12, 71)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:9], "want": [0, 8]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[9:10], "want": []},
+                                     {"id": "b", "tokens": b[:11], "want": [10]}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": b[11:], "want": [0]},
+                                     {"id": "a", "tokens": a[10:], "want": [10]}],
+              "end": ["a", "b"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", d,
+                        "--dtype", "float32", "--out", out, "--max-tokens", "128", "--device", "cpu"],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True,
+                       text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [ln for ln in r.stdout.splitlines() if ln.startswith("done")] == ["done 0", "done 1", "done 2"]
+    orc = oracle(m)
+    ra, rb = orc.forward(a), orc.forward(b)
+    V = m.config.vocab_size
+    got = {i: torch.from_numpy(np.fromfile(os.path.join(out, f"{i}.f32"), dtype="<f4")).view(-1, V)
+           for i in range(3)}
+    check(got[0], ra[[0, 8]])
+    check(got[1], rb[[10]])
+    check(got[2], torch.stack([rb[11], ra[20]]))
+
+
 @pytest.mark.gpu
 def test_bf16_close_to_oracle_and_cut_invariant():
     """bf16 serving: within rounding of the float64 oracle, and the same logits (to rounding)
