@@ -472,3 +472,42 @@ def test_moe_dense_and_grouped_match_oracle(dev, E, top, ff, ffs):
                                    atol=1e-4)
     torch.testing.assert_close(M.moe(hd, wts, gd, dd, E, top, ff, ffs).cpu().to(F64), ref,
                                rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dev", DEVS)
+@pytest.mark.parametrize("pieces,tiled", [([1000], True), ([1000], False), ([150, 1], False),
+                                           ([128, 40, 2], True)])
+def test_attention_far_key_among_hundreds(dev, pieces, tiled):
+    """One early key (position 3) is aligned with the queries near the end of a 200-token prompt,
+    among some two hundred small random keys: rows far away must still find it -- in a prompt, in its
+    portions and when decoded -- and the oracle without that key differs by far more than the
+    tolerance."""
+    from lumen.ops.attention import chunk_sink_attention, write_key_cache
+
+    torch.manual_seed(21)
+    H, G, D, T, bs, chunk, scale = 2, 1, 32, 200, 16, 512, 0.2
+    dtype = torch.bfloat16 if (tiled and dev == "cuda") else torch.float32
+    k = (torch.randn(T, D) * 0.2)
+    q = (torch.randn(T, H * D) * 0.2)
+    d0 = torch.zeros(D)
+    d0[7] = 1.0
+    k[3] += 5 * d0
+    q[190:, :D] += 5 * d0                   # head 0 of the last rows looks for it
+    k, q = k.to(dtype), q.to(dtype)
+    q64, k64 = q.to(F64).view(T, H, D), k.to(F64).view(T, G, D)
+    ref = ref_attention(q64, k64, scale, chunk, 1e-6).reshape(T, H * D)
+    k0 = k64.clone()
+    k0[3, 0] -= 5 * d0.to(F64)
+    without = ref_attention(q64, k0, scale, chunk, 1e-6).reshape(T, H * D)
+    assert float((without[190:, :D] - ref[190:, :D]).abs().max()) > 0.3
+    nb = (T + bs - 1) // bs
+    table = torch.randperm(nb + 1).tolist()[:nb]
+    cache = torch.zeros(nb + 1, bs, G, D, device=DEV, dtype=dtype)
+    got = [torch.zeros(T, H * D, dtype=F64)]
+    for step in cut_steps([T], pieces, 0):
+        sg = seg_of(step, [0], [table], bs, tiled=tiled)
+        write_key_cache(gather(step, [k]).to(DEV), cache, sg.cache_slots)
+        scatter(step, chunk_sink_attention(gather(step, [q]).to(DEV), cache, sg, H, G, D, scale,
+                                           chunk, 1e-6), got)
+    t = dict(rtol=2e-2, atol=2e-2) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(got[0], ref, **t)
