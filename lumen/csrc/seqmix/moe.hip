@@ -4,8 +4,8 @@
 //                  the row's `top` largest logits at their places, zero elsewhere).  One wave per
 //                  row: each lane keeps E / 64 logits in registers, `top` rounds of a wave-wide
 //                  arg-max (ties: lowest index).
-//   sm_gated_act   SwiGLU over stacked [gate | up] blocks, expert e's block scaled by the row's
-//                  routing weight; one thread per output element, fp32 math.
+//   sm_gated_act   act(gate) * up over stacked [gate | up] blocks (act: SiLU, ReLU or tanh-GELU),
+//                  expert e's block scaled by the row's routing weight; fp32 math.
 //   sm_write_k     rows of the key projection into the paged key cache by slot.
 #include "seqmix.h"
 
@@ -14,6 +14,11 @@ using namespace lumen;
 namespace {
 
 constexpr int kMaxPerLane = 16;   // experts <= 1024
+
+// the gate's activation: 0 SiLU, 1 ReLU, 2 tanh-GELU
+__device__ __forceinline__ float gate_act(float g, int act) {
+  return act == 0 ? silu_f(g) : act == 1 ? fmaxf(g, 0.f) : gelu_tanh_f(g);
+}
 
 __global__ void __launch_bounds__(256)
 route_topk_kernel(const float* __restrict__ z, float* __restrict__ out, int T, int E, int top) {
@@ -61,7 +66,8 @@ route_topk_kernel(const float* __restrict__ z, float* __restrict__ out, int T, i
 
 template <typename T>
 __global__ void gated_act_kernel(const T* __restrict__ gu, const float* __restrict__ wts,
-                                 T* __restrict__ out, int Tn, int E, int ff, int ffs) {
+                                 T* __restrict__ out, int Tn, int E, int ff, int ffs,
+                                 int act) {
   const int in_w = E * 2 * ff + 2 * ffs, out_w = E * ff + ffs;
   const long long n = (long long)Tn * out_w;
   for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < n;
@@ -79,7 +85,7 @@ __global__ void gated_act_kernel(const T* __restrict__ gu, const float* __restri
       g = to_f32(row[E * 2 * ff + q]);
       u = to_f32(row[E * 2 * ff + ffs + q]);
     }
-    out[i] = from_f32<T>(w == 0.f ? 0.f : silu_f(g) * u * w);
+    out[i] = from_f32<T>(w == 0.f ? 0.f : gate_act(g, act) * u * w);
   }
 }
 
@@ -87,7 +93,7 @@ __global__ void gated_act_kernel(const T* __restrict__ gu, const float* __restri
 template <typename T>
 __global__ void __launch_bounds__(256)
 gated_act_v8(const T* __restrict__ gu, const float* __restrict__ wts, T* __restrict__ out, int Tn,
-             int E, int ff, int ffs) {
+             int E, int ff, int ffs, int act) {
   const int in_w = E * 2 * ff + 2 * ffs, out_w = E * ff + ffs;
   const int c = 8 * (blockIdx.x * 256 + threadIdx.x);
   if (c >= out_w) return;
@@ -111,7 +117,7 @@ gated_act_v8(const T* __restrict__ gu, const float* __restrict__ wts, T* __restr
       load8<T>(row + goff, g);
       load8<T>(row + uoff, u);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) o[j] = silu_f(g[j]) * u[j] * w;
+      for (int j = 0; j < 8; ++j) o[j] = gate_act(g[j], act) * u[j] * w;
     }
     store8<T>(out + (long long)t * out_w + c, o);
   }
@@ -146,19 +152,21 @@ hipError_t sm_route_topk(const float* z, float* out, int T, int E, int top, hipS
 }
 
 hipError_t sm_gated_act(int dt, const void* gu, const float* wts, void* out, int T, int E, int ff,
-                        int ffs, hipStream_t st) {
+                        int ffs, int act, hipStream_t st) {
   const long long n = (long long)T * (E * ff + ffs);
   if (n == 0) return hipSuccess;
   if (E > 0 && wts == nullptr) return hipErrorInvalidValue;
   if (ff % 8 == 0 && ffs % 8 == 0 && (dt == kBF16 || dt == kF16)) {
     const dim3 grid(((E * ff + ffs) / 8 + 255) / 256, T < 65535 ? T : 65535);
     if (dt == kBF16)
-      gated_act_v8<bf16><<<grid, 256, 0, st>>>((const bf16*)gu, wts, (bf16*)out, T, E, ff, ffs);
+      gated_act_v8<bf16><<<grid, 256, 0, st>>>((const bf16*)gu, wts, (bf16*)out, T, E, ff, ffs,
+                                                 act);
     else
-      gated_act_v8<fp16><<<grid, 256, 0, st>>>((const fp16*)gu, wts, (fp16*)out, T, E, ff, ffs);
+      gated_act_v8<fp16><<<grid, 256, 0, st>>>((const fp16*)gu, wts, (fp16*)out, T, E, ff, ffs,
+                                                 act);
     return hipGetLastError();
   }
-#define CALL(TT) gated_act_kernel<TT><<<grid_for(n), 256, 0, st>>>((const TT*)gu, wts, (TT*)out, T, E, ff, ffs)
+#define CALL(TT) gated_act_kernel<TT><<<grid_for(n), 256, 0, st>>>((const TT*)gu, wts, (TT*)out, T, E, ff, ffs, act)
   SM_DISPATCH(dt, CALL)
 #undef CALL
   return hipGetLastError();

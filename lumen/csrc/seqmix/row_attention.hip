@@ -1,0 +1,396 @@
+// Causal attention of one row against paged caches, with everything between the dot product
+// and the softmax as parameters, and the kernels that prepare its operands:
+//
+//   sm_rotate_heads     interleaved rotary, in place: the pair (x[2i], x[2i+1]) of every head's
+//                       slice [off, off + dims) turns by the angle position * inv_freq[i]
+//   sm_latent_write     a latent-attention layer's cached row: [ RMS-normed latent | shared key
+//                       part, rotated ] from the down projection's output into the paged cache
+//   sm_head_norm_write  q / k RMS norm per head with a weight shared by the heads: q in place,
+//                       normed k and plain v into their paged caches
+//   sm_row_attn         for every row t at position p and every query head h
+//        s_h(j)  = (q1_h . k_g(j)[0:D1] + q2_h . k_g(j)[D1:D1+D2]) * scale * temp(p)
+//        s_h(j) <- cap * tanh(s_h(j) / cap)                       (cap > 0)
+//        s_h(j) <- s_h(j) - r1_h * log(1 + r2_h * (p - j))        (r1 given)
+//        s_h(j) <- sum_h' talk[h, h'] s_h'(j)                     (talk given)
+//        o_h     = sum_{j <= p} exp(s_h(j)) v_g(j) / (sum_{j <= p} exp(s_h(j)) + exp(sink_h))
+//     with temp(p) = 1 + tcoef * log(floor((p + 1) / tevery) + 1), g = h / (H / G), and the
+//     exp(sink_h) term only when a sink is given.  The query may come in two parts (two
+//     pointers with their own strides) that face the two parts of a key row; the value cache may
+//     be the key cache itself (a prefix of the key row is the value).  With G = 1 and D2 > 0 this
+//     is attention over a shared compressed key / value row (the query projected into the latent
+//     space beforehand); with G > 1 it is grouped-query attention.
+//
+// One workgroup of four waves per (row, block of HB heads): a row is a row, whether it belongs
+// to a prompt's portion or is a decoded token, so its result cannot depend on how a step was
+// cut.  Keys are visited 64 at a time, lane = key.  The waves share the heads of the block out
+// among themselves (head w, w + 4, ...): a wave scores its heads against the tile, the scores of
+// all heads meet in LDS (double-buffered, one barrier per tile) where the head mixing reads
+// them, then every wave runs the online softmax and the value pass of its own heads; lanes own
+// 8 output channels of one key group in the value pass (16-byte loads).  Scores, weights, sums
+// and angles are fp32; 16-bit types only appear at loads and stores.
+#include "seqmix.h"
+
+using namespace lumen;
+
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kMaxDv = 512;
+
+template <typename T>
+__global__ void rotate_heads_kernel(T* __restrict__ x, long long ldr, long long ldh, int heads,
+                                    int off, int dims, const float* __restrict__ inv_freq,
+                                    const int* __restrict__ positions, long long n) {
+  const int half = dims / 2;
+  for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    const int pr = (int)(i % half);
+    const long long th = i / half;
+    const int h = (int)(th % heads);
+    const long long t = th / heads;
+    const float a = (float)positions[t] * inv_freq[pr];
+    float sn, cs;
+    sincosf(a, &sn, &cs);
+    T* p = x + t * ldr + h * ldh + off + 2 * pr;
+    const float u = to_f32(p[0]), v = to_f32(p[1]);
+    p[0] = from_f32<T>(u * cs - v * sn);
+    p[1] = from_f32<T>(v * cs + u * sn);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+latent_write_kernel(const T* __restrict__ z, long long ldz, const float* __restrict__ wn,
+                    const float* __restrict__ inv_freq, const int* __restrict__ positions,
+                    const long long* __restrict__ slots, T* __restrict__ cache, int Tn, int R,
+                    int Dr, int dims, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * kWaves + (threadIdx.x >> 6);
+  if (t >= Tn) return;
+  const long long s = slots[t];
+  if (s < 0) return;
+  const T* zr = z + (long long)t * ldz;
+  T* dst = cache + s * (R + Dr);
+  float ss = 0.f;
+  for (int c = lane; c < R; c += 64) {
+    const float v = to_f32(zr[c]);
+    ss += v * v;
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.f / sqrtf(ss / (float)R + eps);
+  for (int c = lane; c < R; c += 64) dst[c] = from_f32<T>(to_f32(zr[c]) * inv * wn[c]);
+  const float pos = (float)positions[t];
+  for (int pr = lane; pr < dims / 2; pr += 64) {
+    float sn, cs;
+    sincosf(pos * inv_freq[pr], &sn, &cs);
+    const float u = to_f32(zr[R + 2 * pr]), v = to_f32(zr[R + 2 * pr + 1]);
+    dst[R + 2 * pr] = from_f32<T>(u * cs - v * sn);
+    dst[R + 2 * pr + 1] = from_f32<T>(v * cs + u * sn);
+  }
+  for (int c = dims + lane; c < Dr; c += 64) dst[R + c] = zr[R + c];
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+head_norm_write_kernel(T* __restrict__ qkv, long long ld, const float* __restrict__ wq,
+                       const float* __restrict__ wk, const long long* __restrict__ slots,
+                       T* __restrict__ kcache, T* __restrict__ vcache, int H, int G, int D, int Dv,
+                       float eps) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const long long s = slots[t];
+  T* row = qkv + (long long)t * ld;
+  for (int item = w; item < H + 2 * G; item += kWaves) {
+    if (item < H + G) {
+      const bool is_q = item < H;
+      T* src = row + (long long)item * D;           // q heads, then k heads, are consecutive
+      float ss = 0.f;
+      for (int c = lane; c < D; c += 64) {
+        const float v = to_f32(src[c]);
+        ss += v * v;
+      }
+      ss = wave_sum(ss);
+      const float inv = 1.f / sqrtf(ss / (float)D + eps);
+      if (is_q) {
+        for (int c = lane; c < D; c += 64) src[c] = from_f32<T>(to_f32(src[c]) * inv * wq[c]);
+      } else if (s >= 0) {
+        T* dst = kcache + (s * G + (item - H)) * D;
+        for (int c = lane; c < D; c += 64) dst[c] = from_f32<T>(to_f32(src[c]) * inv * wk[c]);
+      }
+    } else if (s >= 0) {
+      const int g = item - H - G;
+      const T* src = row + (long long)(H + G) * D + (long long)g * Dv;
+      T* dst = vcache + (s * G + g) * Dv;
+      for (int c = lane; c < Dv; c += 64) dst[c] = src[c];
+    }
+  }
+}
+
+template <typename T>
+struct RowAttnArgs {
+  const T* q1; long long q1r, q1h; int D1;
+  const T* q2; long long q2r, q2h; int D2;
+  const T* kc; long long krow;
+  const T* vc; long long vrow; int Dv;
+  T* out; long long our, ouh;
+  const int* tables; int maxb;
+  const int* row_seg; const int* positions;
+  int H, G, HB, bs;
+  float scale, softcap, tcoef; int tevery;
+  const float *r1, *r2, *talk, *sink;
+};
+
+template <typename T, int HPW>
+__global__ void __launch_bounds__(64 * kWaves)
+row_attn_kernel(const RowAttnArgs<T> a) {
+  extern __shared__ float smem[];
+  const int t = blockIdx.x, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int h0 = blockIdx.y * a.HB;
+  const int nh = min(a.HB, a.H - h0);
+  const int Dk = a.D1 + a.D2;
+  const int pos = a.positions[t];
+  const int* tbl = a.tables + (long long)a.row_seg[t] * a.maxb;
+  const int hpg = a.H / a.G;
+  // LDS: queries [HB][Dk] | scores [2][HB][64] | weights [HB][64] | reduction [4][kMaxDv] |
+  // cache rows of the tile's keys [2][64]
+  float* s_q = smem;
+  float* s_sc = s_q + (long long)a.HB * Dk;
+  float* s_p = s_sc + 2 * a.HB * 64;
+  float* s_o = s_p + a.HB * 64;
+  int* s_rb = reinterpret_cast<int*>(s_o + kWaves * kMaxDv);
+
+  for (int i = threadIdx.x; i < nh * Dk; i += 64 * kWaves) {
+    const int hl = i / Dk, d = i % Dk;
+    const int h = h0 + hl;
+    s_q[i] = d < a.D1 ? to_f32(a.q1[(long long)t * a.q1r + (long long)h * a.q1h + d])
+                      : to_f32(a.q2[(long long)t * a.q2r + (long long)h * a.q2h + (d - a.D1)]);
+  }
+  float temp = 1.f;
+  if (a.tevery > 0 && a.tcoef != 0.f)
+    temp = 1.f + a.tcoef * logf((float)((pos + 1) / a.tevery) + 1.f);
+  const float qscale = a.scale * temp;
+
+  float m[HPW], l[HPW], acc[HPW][8], sreg[HPW];
+#pragma unroll
+  for (int i = 0; i < HPW; ++i) {
+    const int hl = w + kWaves * i;
+    const bool sk = a.sink != nullptr && hl < nh;
+    m[i] = sk ? a.sink[h0 + hl] : -INFINITY;     // the sink: a key of score sink_h, no value
+    l[i] = sk ? 1.f : 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[i][e] = 0.f;
+  }
+  const bool kvec = (Dk % 8 == 0) && (a.krow % 8 == 0);
+  const bool vvec = (a.Dv % 8 == 0) && (a.vrow % 8 == 0);
+  const int lpk = vvec ? a.Dv / 8 : 64, kpi = 64 / lpk;
+  const int grp = lane / lpk, part = lane % lpk;
+  __syncthreads();
+
+  int buf = 0;
+  for (int j0 = 0; j0 <= pos; j0 += 64, buf ^= 1) {
+    const int j = j0 + lane;
+    const bool valid = j <= pos;
+    const int rb = valid ? tbl[j / a.bs] * a.bs + j % a.bs : 0;
+    if (w == 0) s_rb[buf * 64 + lane] = rb;
+    const float dist = (float)(pos - j);
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+      const int hl = w + kWaves * i;
+      if (hl >= nh) break;
+      const int h = h0 + hl;
+      float dot = 0.f;
+      if (valid) {
+        const T* kp = a.kc + (long long)rb * a.krow + (long long)(h / hpg) * Dk;
+        const float* qh = s_q + hl * Dk;
+        if (kvec) {
+          for (int d = 0; d < Dk; d += 8) {
+            float kv[8];
+            load8<T>(kp + d, kv);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dot += qh[d + e] * kv[e];
+          }
+        } else {
+          for (int d = 0; d < Dk; ++d) dot += qh[d] * to_f32(kp[d]);
+        }
+      }
+      float s = dot * qscale;
+      if (a.softcap > 0.f) s = a.softcap * tanhf(s / a.softcap);
+      if (a.r1 != nullptr) s -= a.r1[h] * logf(1.f + a.r2[h] * dist);
+      s = valid ? s : 0.f;
+      sreg[i] = s;
+      s_sc[(buf * a.HB + hl) * 64 + lane] = s;
+    }
+    __syncthreads();
+    const int nk = min(64, pos - j0 + 1);
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+      const int hl = w + kWaves * i;
+      if (hl >= nh) break;
+      const int h = h0 + hl;
+      float s = sreg[i];
+      if (a.talk != nullptr) {
+        s = 0.f;
+        for (int g = 0; g < nh; ++g) s += a.talk[h * a.H + h0 + g] * s_sc[(buf * a.HB + g) * 64 + lane];
+      }
+      s = valid ? s : -INFINITY;
+      const float mn = fmaxf(m[i], wave_max(s));          // finite: the tile's first key is valid
+      const float p = valid ? expf(s - mn) : 0.f;
+      const float corr = expf(m[i] - mn);
+      l[i] = l[i] * corr + wave_sum(p);
+      m[i] = mn;
+      s_p[hl * 64 + lane] = p;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[i][e] *= corr;
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      const long long voff = (long long)(h / hpg) * a.Dv;
+      if (vvec) {
+        if (grp < kpi) {
+          for (int jj = grp; jj < nk; jj += kpi) {
+            const float pj = s_p[hl * 64 + jj];
+            float vv[8];
+            load8<T>(a.vc + (long long)s_rb[buf * 64 + jj] * a.vrow + voff + 8 * part, vv);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[i][e] += pj * vv[e];
+          }
+        }
+      } else {
+        for (int jj = 0; jj < nk; ++jj) {
+          const float pj = s_p[hl * 64 + jj];
+          const T* vp = a.vc + (long long)s_rb[buf * 64 + jj] * a.vrow + voff;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int d = lane + 64 * e;
+            if (d < a.Dv) acc[i][e] += pj * to_f32(vp[d]);
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+
+  float* so = s_o + w * kMaxDv;
+#pragma unroll
+  for (int i = 0; i < HPW; ++i) {
+    const int hl = w + kWaves * i;
+    if (hl >= nh) break;
+    const int h = h0 + hl;
+    if (vvec) {
+      // sum the key groups: every group adds its 8 channels into the wave's LDS row in turn
+      for (int d = lane; d < a.Dv; d += 64) so[d] = 0.f;
+      for (int gq = 0; gq < kpi; ++gq) {
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        if (grp == gq) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) so[8 * part + e] += acc[i][e];
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int d = lane + 64 * e;
+        if (d < a.Dv) so[d] = acc[i][e];
+      }
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    }
+    const float inv = 1.f / l[i];
+    T* op = a.out + (long long)t * a.our + (long long)h * a.ouh;
+    for (int d = lane; d < a.Dv; d += 64) op[d] = from_f32<T>(so[d] * inv);
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+inline size_t row_attn_lds(int HB, int Dk) {
+  return sizeof(float) * ((size_t)HB * Dk + 3 * (size_t)HB * 64 + kWaves * kMaxDv) +
+         sizeof(int) * 2 * 64;
+}
+
+template <typename T>
+hipError_t launch_row_attn(const RowAttnArgs<T>& a, int Tn, hipStream_t st) {
+  const int Dk = a.D1 + a.D2;
+  const size_t lds = row_attn_lds(a.HB, Dk);
+  const dim3 grid(Tn, (a.H + a.HB - 1) / a.HB);
+  const int hpw = (a.HB + kWaves - 1) / kWaves;
+  if (hpw <= 1) row_attn_kernel<T, 1><<<grid, 64 * kWaves, lds, st>>>(a);
+  else if (hpw <= 2) row_attn_kernel<T, 2><<<grid, 64 * kWaves, lds, st>>>(a);
+  else if (hpw <= 4) row_attn_kernel<T, 4><<<grid, 64 * kWaves, lds, st>>>(a);
+  else if (hpw <= 8) row_attn_kernel<T, 8><<<grid, 64 * kWaves, lds, st>>>(a);
+  else return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+inline int grid_for(long long n, int block = 256) {
+  const long long g = (n + block - 1) / block;
+  return (int)(g < 1 ? 1 : g > 65535 ? 65535 : g);
+}
+
+}  // namespace
+
+extern "C" {
+
+hipError_t sm_rotate_heads(int dt, void* x, long long ldr, long long ldh, int heads, int off,
+                           int dims, const float* inv_freq, const int* positions, int T,
+                           hipStream_t st) {
+  const long long n = (long long)T * heads * (dims / 2);
+  if (n == 0) return hipSuccess;
+  if (dims % 2) return hipErrorInvalidValue;
+#define CALL(TT) rotate_heads_kernel<TT><<<grid_for(n), 256, 0, st>>>((TT*)x, ldr, ldh, heads, off, dims, inv_freq, positions, n)
+  SM_DISPATCH(dt, CALL)
+#undef CALL
+  return hipGetLastError();
+}
+
+hipError_t sm_latent_write(int dt, const void* z, long long ldz, const float* wn,
+                           const float* inv_freq, const int* positions, const long long* slots,
+                           void* cache, int T, int R, int Dr, int dims, float eps,
+                           hipStream_t st) {
+  if (T == 0) return hipSuccess;
+  if (dims % 2 || dims > Dr) return hipErrorInvalidValue;
+#define CALL(TT) latent_write_kernel<TT><<<(T + kWaves - 1) / kWaves, 256, 0, st>>>((const TT*)z, ldz, wn, inv_freq, positions, slots, (TT*)cache, T, R, Dr, dims, eps)
+  SM_DISPATCH(dt, CALL)
+#undef CALL
+  return hipGetLastError();
+}
+
+hipError_t sm_head_norm_write(int dt, void* qkv, long long ld, const float* wq, const float* wk,
+                              const long long* slots, void* kcache, void* vcache, int T, int H,
+                              int G, int D, int Dv, float eps, hipStream_t st) {
+  if (T == 0) return hipSuccess;
+#define CALL(TT) head_norm_write_kernel<TT><<<T, 256, 0, st>>>((TT*)qkv, ld, wq, wk, slots, (TT*)kcache, (TT*)vcache, H, G, D, Dv, eps)
+  SM_DISPATCH(dt, CALL)
+#undef CALL
+  return hipGetLastError();
+}
+
+// LDS bytes a (HB heads, key size Dk) block needs; the caller picks HB so that this fits 64 KB
+int sm_row_attn_lds(int HB, int Dk) { return (int)row_attn_lds(HB, Dk); }
+
+hipError_t sm_row_attn(int dt, const void* q1, long long q1r, long long q1h, int D1,
+                       const void* q2, long long q2r, long long q2h, int D2, const void* kc,
+                       long long krow, const void* vc, long long vrow, int Dv, void* out,
+                       long long our, long long ouh, const int* tables, int maxb,
+                       const int* row_seg, const int* positions, int T, int H, int G, int HB,
+                       int bs, float scale, float softcap, float tcoef, int tevery,
+                       const float* r1, const float* r2, const float* talk, const float* sink,
+                       hipStream_t st) {
+  if (T == 0) return hipSuccess;
+  if (H % G != 0 || HB < 1 || HB > 8 * kWaves || Dv > kMaxDv || (talk && HB < H) ||
+      (D2 > 0 && q2 == nullptr) || row_attn_lds(HB, D1 + D2) > 65536)
+    return hipErrorInvalidValue;
+#define CALL(TT)                                                                              \
+  {                                                                                           \
+    RowAttnArgs<TT> a{(const TT*)q1, q1r, q1h, D1, (const TT*)q2, q2r, q2h, D2,               \
+                      (const TT*)kc, krow, (const TT*)vc, vrow, Dv, (TT*)out, our, ouh,       \
+                      tables, maxb, row_seg, positions, H, G, HB, bs, scale, softcap, tcoef,  \
+                      tevery, r1, r2, talk, sink};                                            \
+    return launch_row_attn<TT>(a, T, st);                                                     \
+  }
+  SM_DISPATCH(dt, CALL)
+#undef CALL
+  return hipGetLastError();
+}
+
+}  // extern "C"

@@ -1,4 +1,5 @@
-"""Model families: Llama / Llama-2 (7B, 13B, 70B-GQA), OPT (125m) and Gedatar (hybrid stack)."""
+"""Model families: Llama / Llama-2 (7B, 13B, 70B-GQA), OPT (125m), Gedatar (hybrid stack) and
+Dalavik (latent + grouped-query attention stack)."""
 from __future__ import annotations
 
 from typing import Optional
@@ -6,12 +7,14 @@ from typing import Optional
 import torch
 
 from .config import PRESETS, ModelConfig, checkpoint_dir, get_config  # noqa: F401
+from .dalavik import DalavikForCausalLM  # noqa: F401
 from .gedatar import GedatarForCausalLM  # noqa: F401
 from .llama import LlamaForCausalLM  # noqa: F401
 from .opt import OPTForCausalLM  # noqa: F401
 
 
-MODEL_CLASSES = {"llama": LlamaForCausalLM, "opt": OPTForCausalLM, "gedatar": GedatarForCausalLM}
+MODEL_CLASSES = {"llama": LlamaForCausalLM, "opt": OPTForCausalLM, "gedatar": GedatarForCausalLM,
+                 "dalavik": DalavikForCausalLM}
 
 
 def build_model(name_or_cfg, dtype=torch.bfloat16, device=None, init: str = "auto",

@@ -17,7 +17,7 @@ from typing import Optional
 
 @dataclass
 class ModelConfig:
-    arch: str = "llama"  # "llama" | "opt" | "gedatar"
+    arch: str = "llama"  # "llama" | "opt" | "gedatar" | "dalavik"
     vocab_size: int = 32000
     hidden_size: int = 4096
     intermediate_size: int = 11008
@@ -42,11 +42,16 @@ class ModelConfig:
     # "mlp": {...} | None}, exactly as the checkpoint's config.json lists them
     layer_specs: Optional[list] = None
     canon_taps: int = 0          # taps of the causal depthwise convolution on the mixer input
+    # Dalavik (layer_specs with "latent_attention" | "attention" mixers): groups of the RMS norms
+    # and the per-layer width of the second, per-token embedding (0: the design's side input is off)
+    norm_groups: int = 1
+    token_side_dim: int = 0
 
     @property
     def is_hybrid(self) -> bool:
-        """Layers carry per-sequence recurrent state next to (or instead of) a paged K cache."""
-        return self.arch == "gedatar"
+        """Every layer names its own mixer and keeps its own kind of cache or state; such a stack
+        is served by ``serve.hybrid_runner`` on the step's row segments."""
+        return self.arch in ("gedatar", "dalavik")
 
     @property
     def head_dim(self) -> int:
@@ -63,8 +68,11 @@ class ModelConfig:
     def num_params(self) -> int:
         """Total parameter count (base model, no adapters)."""
         h, v, L = self.hidden_size, self.vocab_size, self.num_hidden_layers
-        if self.arch == "gedatar":
-            from .gedatar import tensor_shapes
+        if self.is_hybrid:
+            if self.arch == "gedatar":
+                from .gedatar import tensor_shapes
+            else:
+                from .dalavik import tensor_shapes
 
             n = 0
             for shape in tensor_shapes(self).values():
@@ -127,9 +135,41 @@ def gedatar_to_dict(cfg: ModelConfig) -> dict:
             "layers": cfg.layer_specs, "eos_token_id": cfg.eos_token_id}
 
 
+def _dalavik_to_config(d: dict) -> ModelConfig:
+    """config.json of a Dalavik checkpoint: {"architecture": "Dalavik", "vocab", "width",
+    "norm": {"eps", "groups"}, "token_side": {"dim"}, "layers": [{"type", "mixer", "mlp"}, ...]}."""
+    layers = d["layers"]
+    if not layers:
+        raise ValueError("a Dalavik config needs at least one layer")
+    for i, L in enumerate(layers):
+        if L.get("type") not in ("latent_attention", "attention"):
+            raise ValueError(f"layer {i}: unknown mixer type {L.get('type')!r}")
+    side = d.get("token_side") or {}
+    return ModelConfig(
+        arch="dalavik", vocab_size=int(d["vocab"]), hidden_size=int(d["width"]),
+        num_hidden_layers=len(layers), rms_norm_eps=float(d["norm"]["eps"]),
+        norm_groups=int(d["norm"].get("groups", 1)), token_side_dim=int(side.get("dim", 0)),
+        layer_specs=layers, intermediate_size=0, num_attention_heads=0, num_key_value_heads=0,
+        max_position_embeddings=1 << 20, tie_word_embeddings=True,
+        bos_token_id=int(d.get("bos_token_id", 0)), eos_token_id=int(d.get("eos_token_id", -1)),
+        pad_token_id=int(d.get("pad_token_id", 0)), name=d.get("_name_or_path", "dalavik"))
+
+
+def dalavik_to_dict(cfg: ModelConfig) -> dict:
+    """The checkpoint form of a Dalavik configuration (inverse of ``_dalavik_to_config``)."""
+    d = {"architecture": "Dalavik", "vocab": cfg.vocab_size, "width": cfg.hidden_size,
+         "norm": {"eps": cfg.rms_norm_eps, "groups": cfg.norm_groups},
+         "layers": cfg.layer_specs, "eos_token_id": cfg.eos_token_id}
+    if cfg.token_side_dim:
+        d["token_side"] = {"dim": cfg.token_side_dim}
+    return d
+
+
 def _hf_to_config(d: dict) -> ModelConfig:
     if d.get("architecture") == "Gedatar":
         return _gedatar_to_config(d)
+    if d.get("architecture") == "Dalavik":
+        return _dalavik_to_config(d)
     mt = d.get("model_type", "llama")
     if mt == "opt":
         return ModelConfig(
@@ -220,6 +260,31 @@ PRESETS = {
             {"type": "attention", "mixer": {"heads": 2, "kv_heads": 2, "dim": 64, "vdim": 64,
                                             "scale": 0.1, "mask": {"size": 40}},
              "mlp": {"kind": "dense", "ff": 160}}]),
+    # latent attention (one layer borrowing another's cache) + grouped-query attention with
+    # temperature, soft cap, distance bias, head mixing and sink; grouped norms; token side input
+    "tiny-dalavik": dict(
+        arch="dalavik", vocab_size=288, hidden_size=96, num_hidden_layers=4, rms_norm_eps=1e-5,
+        norm_groups=3, token_side_dim=8, intermediate_size=0, num_attention_heads=0,
+        num_key_value_heads=0, max_position_embeddings=1 << 20, eos_token_id=-1,
+        tie_word_embeddings=True, name="tiny-dalavik", layer_specs=[
+            {"type": "attention", "mixer": {"heads": 6, "kv_heads": 2, "dim": 24, "vdim": 16,
+                                            "scale": 0.2, "softcap": 12.0,
+                                            "q_temp": {"coef": 0.25, "every": 20}},
+             "mlp": {"kind": "dense", "ff": 160}},
+            {"type": "latent_attention", "mixer": {"heads": 3, "dim": 24, "rot_dim": 8,
+                                                   "vdim": 40, "kv_rank": 32, "q_rank": 48,
+                                                   "scale": 0.15,
+                                                   "rot": {"base": 5000.0, "dims": 8}},
+             "mlp": None},
+            {"type": "latent_attention", "mixer": {"heads": 5, "dim": 16, "rot_dim": 8,
+                                                   "vdim": 24, "kv_rank": 32, "q_rank": 40,
+                                                   "scale": 0.2, "kv_from": 1,
+                                                   "rot": {"base": 5000.0, "dims": 8}},
+             "mlp": {"kind": "dense", "ff": 128}},
+            {"type": "attention", "mixer": {"heads": 2, "kv_heads": 1, "dim": 32, "vdim": 48,
+                                            "scale": 0.18, "softcap": 30.0,
+                                            "q_temp": {"coef": 0.1, "every": 7}},
+             "mlp": {"kind": "dense", "ff": 96}}]),
     "tiny-opt": dict(arch="opt", vocab_size=512, hidden_size=64, intermediate_size=256,
                      ffn_dim=256, num_hidden_layers=2, num_attention_heads=4,
                      num_key_value_heads=4, max_position_embeddings=256, word_embed_proj_dim=64,

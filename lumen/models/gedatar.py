@@ -23,9 +23,9 @@ import math
 from typing import Dict, Tuple
 
 import torch
-import torch.nn as nn
 
 from .config import ModelConfig
+from .named import NamedTensorModel
 
 MIXERS = ("attention", "wkv", "general_delta")
 # general_delta's decay is exp(-DELTA_DECAY * sigmoid(.)): the design fixes the constant
@@ -122,36 +122,13 @@ def validate(cfg: ModelConfig) -> None:
         raise ValueError(f"canon.taps must be in [1, 16], got {cfg.canon_taps}")
 
 
-def _key(name: str) -> str:
-    return name.replace(".", "/")
-
-
-class GedatarForCausalLM(nn.Module):
+class GedatarForCausalLM(NamedTensorModel):
     supports_packing = False
 
     def __init__(self, config: ModelConfig, dtype=torch.bfloat16, device=None,
                  decay_rank: int = DEFAULT_DECAY_RANK):
-        super().__init__()
         validate(config)
-        self.config = config
-        self.dtype = dtype
-        self.tensors = nn.ParameterDict()
-        for name, shape in tensor_shapes(config, decay_rank).items():
-            self.tensors[_key(name)] = nn.Parameter(
-                torch.empty(shape, dtype=dtype, device=device), requires_grad=False)
-
-    # ---- tensors by their checkpoint names -------------------------------------------------
-    def tensor(self, name: str) -> torch.Tensor:
-        return self.tensors[_key(name)]
-
-    def tensor_names(self):
-        return [k.replace("/", ".") for k in self.tensors.keys()]
-
-    def has(self, name: str) -> bool:
-        return _key(name) in self.tensors
-
-    def replace_tensor(self, name: str, value: torch.Tensor) -> None:
-        self.tensors[_key(name)] = nn.Parameter(value, requires_grad=False)
+        super().__init__(config, tensor_shapes(config, decay_rank), dtype, device)
 
     @torch.no_grad()
     def init_weights(self, std: float = 0.02, seed: int = 0):

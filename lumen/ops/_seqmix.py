@@ -32,7 +32,13 @@ SIGNATURES = {
     "sm_chunk_attn": "iplpppippiiiiiffii",
     "sm_chunk_attn_tiles": "iplpppipippiiiiffiii",
     "sm_route_topk": "ppiii",
-    "sm_gated_act": "ipppiiii",
+    "sm_gated_act": "ipppiiiii",
+    "sm_group_rms": "iiplpppliiif",
+    "sm_gate_rows": "iplplpiipi",
+    "sm_rotate_heads": "iplliiippi",
+    "sm_latent_write": "iplpppppiiiif",
+    "sm_head_norm_write": "iplpppppiiiiif",
+    "sm_row_attn": "i" "plli" "plli" "pl" "pli" "pll" "pi" "pp" "iiiii" "fffi" "pppp",
 }
 
 
@@ -53,6 +59,8 @@ def _load():
             fn.restype = ctypes.c_int
         lib.sm_chunk_attn_tiles_ok.argtypes = [ctypes.c_int, ctypes.c_int]
         lib.sm_chunk_attn_tiles_ok.restype = ctypes.c_int
+        lib.sm_row_attn_lds.argtypes = [ctypes.c_int, ctypes.c_int]
+        lib.sm_row_attn_lds.restype = ctypes.c_int
         _lib = lib
     except Exception as e:  # pragma: no cover - depends on build state
         _err = e
@@ -80,6 +88,11 @@ DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 def tiles_ok(dt: int, D: int) -> bool:
     """Does the matrix-core prefill attention have a kernel for this dtype code / head size?"""
     return bool(_load().sm_chunk_attn_tiles_ok(dt, D))
+
+
+def row_attn_lds(HB: int, Dk: int) -> int:
+    """LDS bytes the row-attention kernel needs for a block of HB heads with key size Dk."""
+    return int(_load().sm_row_attn_lds(HB, Dk))
 
 
 def _arg(kind, v):

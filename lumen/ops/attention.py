@@ -580,3 +580,180 @@ def chunk_sink_attention(q: torch.Tensor, cache: torch.Tensor, seg, H: int, G: i
              seg.row_seg[Tp:], seg.positions[Tp:], T - Tp, H, G, D, bs, scale, eps, chunk,
              int(sink))
     return out
+
+
+# ---- row attention over paged caches: latent (shared compressed row) and grouped-query ----------
+# One kernel (``csrc/seqmix/row_attention.hip``) serves prompts' portions and decoded rows: a
+# row's position and its segment's block table say which keys it sees.  What stands between the
+# dot product and the softmax is a parameter: a position-dependent query temperature, a tanh soft
+# cap, a logarithmic distance bias per head, a mixing of the heads' scores, a per-head sink in
+# the softmax denominator.  Scores and weights are fp32.
+def latent_write_ref(z, w_norm, inv_freq, positions, slots, cache, R, dims, eps):
+    zf = z.float()
+    c = zf[:, :R]
+    c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * w_norm.float()
+    kr = zf[:, R:].clone()
+    a = positions.float().view(-1, 1) * inv_freq.float().view(1, -1)
+    u, v = kr[:, 0:dims:2].clone(), kr[:, 1:dims:2].clone()
+    kr[:, 0:dims:2] = u * torch.cos(a) - v * torch.sin(a)
+    kr[:, 1:dims:2] = v * torch.cos(a) + u * torch.sin(a)
+    ok = slots >= 0
+    cache.view(-1, cache.shape[-1])[slots[ok]] = torch.cat([c, kr], 1)[ok].to(cache.dtype)
+
+
+def latent_write(z: torch.Tensor, w_norm: torch.Tensor, inv_freq: torch.Tensor,
+                 positions: torch.Tensor, slots: torch.Tensor, cache: torch.Tensor, R: int,
+                 dims: int, eps: float) -> None:
+    """Rows of a latent-attention layer's down projection z [T, R + Dr] into the paged cache
+    [blocks, block, R + Dr] at ``slots`` (int64; -1 skips): the first R columns RMS-normed with
+    ``w_norm``, the rest (the key part all heads share) rotated on its first ``dims`` columns."""
+    from ._seqmix import DT, call, use_seqmix
+
+    Dr = z.shape[1] - R
+    if cache.shape[-1] != R + Dr or dims > Dr or dims % 2:
+        raise ValueError(f"latent row {R}+{Dr} (rotary {dims}) does not fit cache rows of "
+                         f"{cache.shape[-1]}")
+    if not use_seqmix(z):
+        return latent_write_ref(z, w_norm, inv_freq, positions, slots, cache, R, dims, eps)
+    assert z.stride(1) == 1 and cache.is_contiguous() and cache.dtype == z.dtype
+    call("sm_latent_write", DT[z.dtype], z, z.stride(0), w_norm, inv_freq, positions, slots, cache,
+         z.shape[0], R, Dr, dims, eps)
+
+
+def head_norm_write_ref(qkv, wq, wk, slots, kcache, vcache, H, G, D, Dv, eps):
+    T = qkv.shape[0]
+
+    def unit(x):
+        x = x.float()
+        return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+
+    q = unit(qkv[:, :H * D].reshape(T, H, D)) * wq.float()
+    k = unit(qkv[:, H * D:(H + G) * D].reshape(T, G, D)) * wk.float()
+    qkv[:, :H * D] = q.reshape(T, H * D).to(qkv.dtype)
+    ok = slots >= 0
+    kcache.view(-1, G, D)[slots[ok]] = k[ok].to(kcache.dtype)
+    vcache.view(-1, G, Dv)[slots[ok]] = qkv[:, (H + G) * D:].reshape(T, G, Dv)[ok].to(vcache.dtype)
+
+
+def head_norm_write(qkv: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, slots: torch.Tensor,
+                    kcache: torch.Tensor, vcache: torch.Tensor, H: int, G: int, D: int, Dv: int,
+                    eps: float) -> None:
+    """qkv [T, H * D + G * D + G * Dv] (a fused projection's output): every query head and key
+    head is RMS-normed over its D entries with the weight ``wq`` / ``wk`` [D] shared by the heads;
+    q is replaced in place, the normed keys and the values go to their paged caches
+    [blocks, block, G, D] / [blocks, block, G, Dv] at ``slots`` (int64; -1 skips)."""
+    from ._seqmix import DT, call, use_seqmix
+
+    if qkv.shape[1] != (H + G) * D + G * Dv:
+        raise ValueError(f"qkv has {qkv.shape[1]} columns, expected {(H + G) * D + G * Dv}")
+    if not use_seqmix(qkv):
+        return head_norm_write_ref(qkv, wq, wk, slots, kcache, vcache, H, G, D, Dv, eps)
+    assert qkv.stride(1) == 1 and kcache.is_contiguous() and vcache.is_contiguous()
+    assert kcache.dtype == qkv.dtype and vcache.dtype == qkv.dtype
+    assert tuple(kcache.shape[2:]) == (G, D) and tuple(vcache.shape[2:]) == (G, Dv)
+    call("sm_head_norm_write", DT[qkv.dtype], qkv, qkv.stride(0), wq, wk, slots, kcache, vcache,
+         qkv.shape[0], H, G, D, Dv, eps)
+
+
+def row_attention_ref(q1, q2, kcache, vcache, Dv, out, seg, H, G, scale, softcap=0.0,
+                      q_temp=None, r1=None, r2=None, talk=None, sink=None):
+    T = q1.shape[0]
+    D1 = q1.shape[2]
+    D2 = q2.shape[2] if q2 is not None else 0
+    Dk = D1 + D2
+    bs = kcache.shape[1]
+    krows = kcache.reshape(kcache.shape[0] * bs, -1)
+    vrows = vcache.reshape(vcache.shape[0] * bs, -1)
+    q = q1.float() if q2 is None else torch.cat([q1.float(), q2.float()], -1)    # [T, H, Dk]
+    row_seg, pos = seg.row_seg.tolist(), seg.positions.tolist()
+    hg = torch.arange(H, device=q.device) // (H // G)
+    for t in range(T):
+        p = pos[t]
+        js = torch.arange(0, p + 1, device=q.device)
+        tbl = seg.tables[row_seg[t]].long()
+        rows = tbl[js // bs] * bs + js % bs
+        k = krows[rows][:, :G * Dk].float().view(-1, G, Dk)[:, hg]              # [n, H, Dk]
+        v = vrows[rows].float()
+        v = (v[:, :G * Dv].view(-1, G, Dv) if G > 1 or vrows.shape[1] == Dv
+             else v[:, :Dv].view(-1, 1, Dv))[:, hg]                             # [n, H, Dv]
+        temp = 1.0
+        if q_temp is not None and q_temp[0] != 0.0 and q_temp[1] > 0:
+            temp = 1.0 + q_temp[0] * math.log((p + 1) // q_temp[1] + 1.0)
+        s = torch.einsum("hd,nhd->hn", q[t], k) * (scale * temp)
+        if softcap and softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
+        if r1 is not None:
+            d = (p - js).float()
+            s = s - r1.float().view(H, 1) * torch.log(1.0 + r2.float().view(H, 1) * d)
+        if talk is not None:
+            s = talk.float() @ s
+        m = s.max(-1, keepdim=True).values
+        if sink is not None:
+            m = torch.maximum(m, sink.float().view(H, 1))
+        e = torch.exp(s - m)
+        den = e.sum(-1, keepdim=True)
+        if sink is not None:
+            den = den + torch.exp(sink.float().view(H, 1) - m)
+        out[t] = torch.einsum("hn,nhd->hd", e / den, v).to(out.dtype)
+    return out
+
+
+def _heads_per_block(H: int, Dk: int, need_all: bool) -> int:
+    """Heads one workgroup of the row kernel takes: as many as its LDS (64 KB) holds, at most 32;
+    a power of two unless all H are needed (head mixing)."""
+    from ._seqmix import row_attn_lds
+
+    if need_all:
+        if H > 32 or row_attn_lds(H, Dk) > 65536:
+            raise ValueError(f"head mixing over {H} heads of key size {Dk} does not fit the "
+                             "attention kernel (at most 32 heads, 64 KB of LDS)")
+        return H
+    hb = 1
+    while hb * 2 <= min(H, 16) and row_attn_lds(hb * 2, Dk) <= 65536:
+        hb *= 2
+    return hb
+
+
+def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Tensor,
+                  vcache: torch.Tensor, Dv: int, out: torch.Tensor, seg, H: int, G: int,
+                  scale: float, softcap: float = 0.0, q_temp=None, r1=None, r2=None, talk=None,
+                  sink=None) -> torch.Tensor:
+    """Causal attention of every row of a step against paged caches.
+
+    q1 [T, H, D1] and (optionally) q2 [T, H, D2] are views with arbitrary row / head strides;
+    a key row is ``kcache[block, i, g * Dk : (g + 1) * Dk]`` with Dk = D1 + D2 (q1 faces its
+    first D1 entries, q2 the rest); a value row is ``vcache[block, i, g * Dv : (g + 1) * Dv]``
+    -- ``vcache`` may be ``kcache`` itself (G = 1: the value is a prefix of the key row).
+    ``out`` [T, H, Dv] is a view with arbitrary row / head strides.  The step's own keys must
+    already be in the cache.  ``q_temp`` = (coef, every): the score of a row at position p is
+    multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).  ``softcap`` > 0: s <- cap *
+    tanh(s / cap).  ``r1``, ``r2`` [H]: s <- s - r1 * ln(1 + r2 * distance).  ``talk`` [H, H]:
+    the heads' scores are mixed, s_h <- sum_g talk[h, g] s_g.  ``sink`` [H]: exp(sink_h) joins
+    the softmax denominator."""
+    from ._seqmix import DT, call, use_seqmix
+
+    T, _, D1 = q1.shape
+    D2 = q2.shape[2] if q2 is not None else 0
+    Dk = D1 + D2
+    if H % G:
+        raise ValueError(f"{H} heads are not a multiple of {G} key/value heads")
+    if not use_seqmix(q1):
+        return row_attention_ref(q1, q2, kcache, vcache, Dv, out, seg, H, G, scale, softcap,
+                                 q_temp, r1, r2, talk, sink)
+    if Dv > 512:
+        raise ValueError(f"value size {Dv} > 512 is not supported")
+    assert kcache.is_contiguous() and vcache.is_contiguous() and kcache.dtype == q1.dtype
+    assert q1.stride(2) == 1 and out.stride(2) == 1 and (q2 is None or q2.stride(2) == 1)
+    krow = kcache.shape[2:].numel()
+    vrow = vcache.shape[2:].numel()
+    assert krow >= G * Dk and vrow >= G * Dv
+    for f in (r1, r2, talk, sink):
+        assert f is None or (f.dtype == torch.float32 and f.is_contiguous())
+    HB = _heads_per_block(H, Dk, talk is not None)
+    coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp is not None else (0.0, 0)
+    call("sm_row_attn", DT[q1.dtype], q1, q1.stride(0), q1.stride(1), D1,
+         q2, q2.stride(0) if q2 is not None else 0, q2.stride(1) if q2 is not None else 0, D2,
+         kcache, krow, vcache, vrow, Dv, out, out.stride(0), out.stride(1),
+         seg.tables, seg.tables.shape[1], seg.row_seg, seg.positions, T, H, G, HB,
+         kcache.shape[1], scale, float(softcap or 0.0), coef, every, r1, r2, talk, sink)
+    return out

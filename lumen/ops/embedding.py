@@ -20,3 +20,29 @@ def embedding(ids: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         native().embedding(weight, flat, out)
         return out.view(*ids.shape, weight.shape[1])
     return F.embedding(ids, weight)
+
+
+def gated_token_slice_ref(z, table, tokens, col0):
+    dim = z.shape[1]
+    e = table[tokens][:, col0:col0 + dim].float()
+    return (F.gelu(z.float(), approximate="tanh") * e).to(z.dtype)
+
+
+def gated_token_slice(z: torch.Tensor, table: torch.Tensor, tokens: torch.Tensor,
+                      col0: int) -> torch.Tensor:
+    """gelu_tanh(z) * table[tokens, col0 : col0 + dim] for z [T, dim]: a column slice of a second
+    per-token embedding, gated by a projection of the residual stream (gather and activation in
+    one pass; HIP ``csrc/seqmix/rms_group.hip``)."""
+    from ._seqmix import DT, call, use_seqmix
+
+    if not use_seqmix(z):
+        return gated_token_slice_ref(z, table, tokens, col0)
+    assert z.stride(1) == 1 and table.stride(1) == 1 and table.dtype == z.dtype
+    assert tokens.dtype == torch.int64 and tokens.is_contiguous()
+    T, dim = z.shape
+    if col0 < 0 or col0 + dim > table.shape[1]:
+        raise ValueError(f"columns [{col0}, {col0 + dim}) outside a table of {table.shape[1]}")
+    out = torch.empty(T, dim, dtype=z.dtype, device=z.device)
+    call("sm_gate_rows", DT[z.dtype], z, z.stride(0), table, table.stride(0), tokens, col0, dim,
+         out, T)
+    return out

@@ -45,31 +45,36 @@ def route_topk(z: torch.Tensor, top: int) -> torch.Tensor:
     return out
 
 
-def gated_act_ref(gu, wts, E, ff, ffs):
+GATE_ACTS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+_ACT_FN = {"silu": F.silu, "relu": F.relu, "gelu_tanh": lambda z: F.gelu(z, approximate="tanh")}
+
+
+def gated_act_ref(gu, wts, E, ff, ffs, act="silu"):
     T = gu.shape[0]
+    fn = _ACT_FN[act]
     parts = []
     if E:
         g = gu[:, :E * 2 * ff].float().view(T, E, 2, ff)
-        parts.append((F.silu(g[:, :, 0]) * g[:, :, 1] * wts.float()[:, :, None]).reshape(T, E * ff))
+        parts.append((fn(g[:, :, 0]) * g[:, :, 1] * wts.float()[:, :, None]).reshape(T, E * ff))
     if ffs:
         s = gu[:, E * 2 * ff:].float().view(T, 2, ffs)
-        parts.append(F.silu(s[:, 0]) * s[:, 1])
+        parts.append(fn(s[:, 0]) * s[:, 1])
     return torch.cat(parts, 1).to(gu.dtype)
 
 
 def gated_act(gu: torch.Tensor, wts: Optional[torch.Tensor], E: int, ff: int,
-              ffs: int) -> torch.Tensor:
-    """SwiGLU over stacked [gate | up] blocks: ``gu`` [T, E * 2 * ff + 2 * ffs] holds E expert
-    blocks (gate rows then up rows, ff each) and one unweighted block of ffs (a dense
-    feed-forward, or the shared expert); expert e's activation is scaled by ``wts[:, e]``.
-    Returns [T, E * ff + ffs]."""
+              ffs: int, act: str = "silu") -> torch.Tensor:
+    """act(gate) * up over stacked [gate | up] blocks (``act``: silu, i.e. SwiGLU, relu or
+    gelu_tanh): ``gu`` [T, E * 2 * ff + 2 * ffs] holds E expert blocks (gate rows then up rows,
+    ff each) and one unweighted block of ffs (a dense feed-forward, or the shared expert);
+    expert e's activation is scaled by ``wts[:, e]``.  Returns [T, E * ff + ffs]."""
     from ._seqmix import DT, call, use_seqmix
 
     if not use_seqmix(gu):
-        return gated_act_ref(gu, wts, E, ff, ffs)
+        return gated_act_ref(gu, wts, E, ff, ffs, act)
     assert gu.is_contiguous() and gu.shape[1] == E * 2 * ff + 2 * ffs
     out = torch.empty(gu.shape[0], E * ff + ffs, dtype=gu.dtype, device=gu.device)
-    call("sm_gated_act", DT[gu.dtype], gu, wts, out, gu.shape[0], E, ff, ffs)
+    call("sm_gated_act", DT[gu.dtype], gu, wts, out, gu.shape[0], E, ff, ffs, GATE_ACTS[act])
     return out
 
 

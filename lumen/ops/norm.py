@@ -126,3 +126,59 @@ def dyt_residual(x: torch.Tensor, y: torch.Tensor, post, pre=None, out_dtype=Non
     call("sm_dyt_residual", DT[y.dtype], DT[out_dtype], x, y, post[0], post[1], post[2], h,
          p[0], p[1], p[2], x.shape[0], x.shape[1])
     return x, h
+
+
+# ---- RMS norm in groups ------------------------------------------------------------------------
+# The row is split into ``groups`` equal consecutive parts and each part is divided by its own
+# sqrt(mean(part^2) + eps); the whole row is then multiplied by w (groups = 1: the ordinary RMS
+# norm with a plain weight).  fp32 throughout; only a stored result is rounded.
+# (HIP: ``csrc/seqmix/rms_group.hip``.)
+def group_rms_norm_ref(x, w, groups, eps, out_dtype=None):
+    shp = x.shape
+    g = x.float().reshape(*shp[:-1], groups, shp[-1] // groups)
+    y = (g / torch.sqrt((g * g).mean(-1, keepdim=True) + eps)).reshape(shp) * w.float()
+    return y.to(out_dtype or x.dtype)
+
+
+def group_rms_norm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float,
+                   out_dtype=None) -> torch.Tensor:
+    """Group RMS norm of the rows of ``x`` [rows, W] (fp32 or 16-bit; the rows may be a column
+    slice of a wider buffer) with the fp32 weight ``w`` [W], stored in ``out_dtype``."""
+    from ._seqmix import DT, call, use_seqmix
+
+    out_dtype = out_dtype or x.dtype
+    if x.shape[-1] % groups:
+        raise ValueError(f"width {x.shape[-1]} is not a multiple of {groups} groups")
+    if not use_seqmix(x):
+        return group_rms_norm_ref(x, w, groups, eps, out_dtype)
+    assert x.dim() == 2 and x.stride(1) == 1 and w.dtype == torch.float32
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    call("sm_group_rms", DT[x.dtype], DT[out_dtype], x, x.stride(0), w, None, out, out.stride(0),
+         x.shape[0], x.shape[1], groups, eps)
+    return out
+
+
+def group_rms_residual_ref(x, y, w, groups, eps, cast=None):
+    x.add_(group_rms_norm_ref(y, w, groups, eps, torch.float32))
+    return x, (x.to(cast) if cast is not None and cast != x.dtype else None)
+
+
+def group_rms_residual(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, groups: int,
+                       eps: float, cast=None):
+    """The fp32 residual stream ``x`` [T, W] takes a sublayer's normed output in place,
+    x += group_rms_norm(y) * w, and -- fused, when ``cast`` is a 16-bit dtype -- the new stream is
+    also returned rounded to ``cast`` (what the next sublayer's GEMMs read).  Returns
+    (x, x in ``cast`` or None)."""
+    from ._seqmix import DT, call, use_seqmix
+
+    if x.shape[-1] % groups:
+        raise ValueError(f"width {x.shape[-1]} is not a multiple of {groups} groups")
+    if not use_seqmix(x):
+        return group_rms_residual_ref(x, y, w, groups, eps, cast)
+    assert x.dtype == torch.float32 and x.is_contiguous() and y.stride(1) == 1
+    xb = None
+    if cast is not None and cast != torch.float32:
+        xb = torch.empty(x.shape, dtype=cast, device=x.device)
+    call("sm_group_rms", DT[y.dtype], DT[cast if xb is not None else torch.float32], y,
+         y.stride(0), w, x, xb, x.shape[1], x.shape[0], x.shape[1], groups, eps)
+    return x, xb

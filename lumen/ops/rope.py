@@ -156,3 +156,49 @@ def rope_qkv_(qkv: torch.Tensor, pos: torch.Tensor, nh: int, nkv: int, D: int, c
     p = pos.long()
     rot = _rotate_ref(view, cos_t[p][:, None], sin_t[p][:, None])
     return torch.cat([rot.reshape(T, -1), out[:, (nh + nkv) * D:]], 1)
+
+
+# ---- interleaved rotary at arbitrary positions ---------------------------------------------------
+# The pair (x[2i], x[2i + 1]) of a head's slice [off, off + dims) turns by the angle
+# position * base^(-2i / dims); what lies outside the slice passes unchanged.  The frequencies are
+# computed once on the host in float64 and rounded to fp32; the angle and the rotation are fp32.
+_INV_FREQ: Dict[tuple, torch.Tensor] = {}
+
+
+def interleaved_inv_freq(dims: int, base: float, device) -> torch.Tensor:
+    key = (int(dims), float(base), str(device))
+    t = _INV_FREQ.get(key)
+    if t is None:
+        t = torch.tensor([float(base) ** (-2.0 * i / dims) for i in range(dims // 2)],
+                         dtype=torch.float64).float().to(device)
+        _INV_FREQ[key] = t
+    return t
+
+
+def rotate_interleaved_ref(x, positions, heads, head_stride, off, dims, inv_freq):
+    T = x.shape[0]
+    a = positions.float().view(T, 1, 1) * inv_freq.float().view(1, 1, -1)
+    cs, sn = torch.cos(a), torch.sin(a)
+    v = torch.as_strided(x, (T, heads, dims), (x.stride(0), head_stride, 1),
+                         x.storage_offset() + off)
+    u0, u1 = v[..., 0::2].float(), v[..., 1::2].float()
+    r0, r1 = u0 * cs - u1 * sn, u1 * cs + u0 * sn
+    v[..., 0::2] = r0.to(x.dtype)
+    v[..., 1::2] = r1.to(x.dtype)
+    return x
+
+
+def rotate_interleaved_(x: torch.Tensor, positions: torch.Tensor, heads: int, head_stride: int,
+                        off: int, dims: int, inv_freq: torch.Tensor) -> torch.Tensor:
+    """In place: rows of x [T, >= (heads - 1) * head_stride + off + dims] (unit column stride),
+    head h's slice starting at column h * head_stride + off; ``positions`` [T] int32."""
+    from ._seqmix import DT, call, use_seqmix
+
+    if dims % 2:
+        raise ValueError(f"rotary dims must be even, got {dims}")
+    if not use_seqmix(x):
+        return rotate_interleaved_ref(x, positions, heads, head_stride, off, dims, inv_freq)
+    assert x.stride(1) == 1 and positions.dtype == torch.int32
+    call("sm_rotate_heads", DT[x.dtype], x, x.stride(0), head_stride, heads, off, dims, inv_freq,
+         positions, x.shape[0])
+    return x

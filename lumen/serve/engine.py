@@ -161,9 +161,9 @@ class LLMEngine:
         self.hybrid = bool(getattr(model.config, "is_hybrid", False))
         if self.hybrid:
             self._check_hybrid_options()
-            from .hybrid_runner import HybridWeights
+            from .hybrid_runner import WEIGHTS
 
-            self.weights = HybridWeights(model, self.rank, self.tp)
+            self.weights = WEIGHTS[model.config.arch](model, self.rank, self.tp)
         else:
             self.weights = ServeWeights(model, self.rank, self.tp)
         if cfg.kv_cache_dtype not in ("auto", "fp8"):

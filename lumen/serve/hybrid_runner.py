@@ -1,4 +1,10 @@
-"""Serving runner for hybrid stacks (Gedatar): paged key cache + per-sequence recurrent state.
+"""Serving runner for stacks whose layers each name their own mixer (Gedatar, Dalavik): paged
+caches + per-sequence recurrent state.
+
+Two families share the runner, the segments, the block manager and the hipGraph decode; each has
+its weights class (stacked projections, fp32 constants), its caches and its step function:
+Gedatar (``HybridWeights`` / ``HybridState`` / ``run_layers``, described next) and Dalavik
+(``DalavikWeights`` / ``DalavikState``, further down).
 
 One step function for prefill chunks, decode rows and mixtures of both.  The rows of a step are
 cut into segments (``ops.segments.SegBatch``: one per chunk, one per decode row); per layer
@@ -34,11 +40,14 @@ import torch.nn.functional as F
 
 from ..models.config import ModelConfig
 from ..models.gedatar import DELTA_DECAY, DELTA_KEY_EPS
-from ..ops.attention import chunk_sink_attention, write_key_cache
+from ..ops.attention import (chunk_sink_attention, head_norm_write, latent_write, row_attention,
+                             write_key_cache)
 from ..ops.conv import dyt_canon
+from ..ops.embedding import gated_token_slice
 from ..ops.moe import gated_act, moe, route_topk
-from ..ops.norm import dyt, dyt_residual
+from ..ops.norm import dyt, dyt_residual, group_rms_norm, group_rms_residual
 from ..ops.recurrent import delta_scan, token_shift, wkv_scan
+from ..ops.rope import rotate_interleaved_
 from ..ops.segments import SegBatch, whole_sequences
 from .model_runner import ModelRunner, StepInput
 
@@ -116,6 +125,17 @@ class HybridWeights:
                 self.layers.append(L)
 
 
+    # ---- what HybridRunner asks of a family's weights ----------------------------------------
+    def new_state(self, slots: int, num_blocks: int, block_size: int, device):
+        return HybridState(self, slots, num_blocks, block_size, device)
+
+    def run_layers(self, st, tokens, seg, observe=None) -> torch.Tensor:
+        return run_layers(self, st, tokens, seg, observe)
+
+    def head(self, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(dyt(x, self.final, self.dtype), self.lm_head)
+
+
 class HybridState:
     """Per-layer caches of a hybrid model: ``slots`` sequences of recurrent state (+ one spare
     slot for graph padding rows) and ``num_blocks`` pages of keys for the attention layers."""
@@ -141,11 +161,23 @@ class HybridState:
 
 
 def key_bytes_per_token(cfg: ModelConfig, dtype_bytes: int = 2) -> int:
+    """Bytes of paged cache one token takes over all layers."""
+    if cfg.arch == "dalavik":
+        n = 0
+        for L in cfg.layer_specs:
+            m = L["mixer"]
+            if L["type"] == "attention":
+                n += m["kv_heads"] * (m["dim"] + m["vdim"])
+            elif m.get("kv_from") is None:
+                n += m["kv_rank"] + m["rot_dim"]
+        return max(1, n * dtype_bytes)
     return max(1, sum(L["mixer"]["kv_heads"] * L["mixer"]["dim"] for L in cfg.layer_specs
                       if L["type"] == "attention") * dtype_bytes)
 
 
 def state_bytes_per_slot(cfg: ModelConfig) -> int:
+    if cfg.arch == "dalavik":
+        return 0
     n = 0
     for L in cfg.layer_specs:
         n += max(cfg.canon_taps - 1, 0) * cfg.hidden_size
@@ -207,6 +239,192 @@ def run_layers(w: HybridWeights, st: HybridState, tokens: torch.Tensor, seg: Seg
     return x
 
 
+# ---- Dalavik: latent attention + grouped-query attention with score shaping ----------------------
+#
+#   x, xb   the fp32 residual stream and (16-bit serving) its rounded copy that the GEMMs read;
+#           every residual kernel hands both on, so no separate cast pass exists
+#   latent_attention
+#       z  = [W_dq ; W_dkv] xb               one GEMM; a layer that borrows a cache has W_dq only
+#       cache row <- [rms(z_kv[:R]) * w | rotate(z_kv[R:])]                     (latent_write)
+#       q  = W_uq (rms(z_q) * w), its rotated part turned in place               (rotate_interleaved_)
+#       qa = per-head W_uk^T q_plain         the query in the latent space (batched GEMM)
+#       ol = row_attention([qa | q_rot] against the cached row, value = its first R columns)
+#       y  = W_o (per-head W_uv ol)          (batched GEMM into the token-major layout, then GEMM)
+#   attention
+#       qkv = [W_q ; W_k ; W_v] xb + b       one GEMM
+#       q normed in place, normed k and v into their caches                      (head_norm_write)
+#       o  = row_attention(temperature, soft cap, distance bias, head mixing, sink);  y = W_o o
+#   x += gnorm_1(y)                          (group_rms_residual, also the next xb)
+#   x += gnorm_2(W_down (relu(gate) * up))   one [gate ; up] GEMM, fused activation
+#   x += rms(W_proj (gelu_tanh(W_sgate xb) * E[token, slice])) * w               (token side input)
+#
+# fp32: the stream, every norm, angles, scores, softmax; model dtype: GEMMs and what they store.
+# Nothing here is per-sequence state: a sequence's whole memory is its cache blocks.
+@dataclass
+class DalavikLayerW:
+    kind: str                       # latent_attention | attention
+    m: dict                         # the mixer's sizes and constants
+    norm1: torch.Tensor
+    w: Dict[str, torch.Tensor] = field(default_factory=dict)
+    ff: Optional[dict] = None       # gu [2 ff, W], down [W, ff], ff, norm
+    side: Optional[dict] = None     # gate [d, W], proj [W, d], norm [W], col0
+    kv_layer: int = -1              # latent attention: the layer whose cache rows it reads
+
+
+class DalavikWeights:
+    """Inference weights of a DalavikForCausalLM: projections that share an input are stacked
+    into one GEMM, the per-head up projections are laid out for batched GEMMs, norm weights and
+    the attention's per-head constants are fp32."""
+
+    def __init__(self, model, tp_rank: int = 0, tp_size: int = 1):
+        if tp_size != 1:
+            raise NotImplementedError("Dalavik models are served at tensor-parallel size 1")
+        from ..ops.rope import interleaved_inv_freq
+
+        cfg: ModelConfig = model.config
+        self.cfg = cfg
+        t = model.tensor
+        f32 = lambda n: t(n).detach().float().contiguous()  # noqa: E731
+        self.dtype = t("embed").dtype
+        dev = t("embed").device
+        self.embed = t("embed").detach()
+        self.lm_head = self.embed                           # tied
+        self.final = f32("final.norm")
+        self.vocab_shard = cfg.vocab_size
+        sd = cfg.token_side_dim
+        self.side_embed = t("side.embed").detach() if sd else None
+        self.layers: List[DalavikLayerW] = []
+        with torch.no_grad():
+            for i, spec in enumerate(cfg.layer_specs):
+                p, m = f"l{i}.", spec["mixer"]
+                x = p + "mix."
+                L = DalavikLayerW(spec["type"], m, f32(p + "norm1"))
+                if L.kind == "latent_attention":
+                    H, D, Dv, R = m["heads"], m["dim"], m["vdim"], m["kv_rank"]
+                    own = m.get("kv_from") is None
+                    L.kv_layer = i if own else int(m["kv_from"])
+                    L.w["down"] = (torch.cat([t(x + "dq"), t(x + "dkv")], 0).contiguous()
+                                   if own else t(x + "dq").detach())
+                    L.w["dq_norm"] = f32(x + "dq.norm")
+                    if own:
+                        L.w["dkv_norm"] = f32(x + "dkv.norm")
+                    L.w["uq"] = t(x + "uq").detach()
+                    L.w["uk"] = t(x + "uk").detach().view(H, D, R)                   # q_h @ uk[h]
+                    L.w["uvT"] = t(x + "uv").detach().view(H, Dv, R).transpose(1, 2).contiguous()
+                    L.w["inv_freq"] = interleaved_inv_freq(m["rot"]["dims"], m["rot"]["base"], dev)
+                else:
+                    L.w["qkv"] = torch.cat([t(x + n) for n in "qkv"], 0).contiguous()
+                    L.w["qkv_b"] = torch.cat([t(x + n + ".b") for n in "qkv"], 0).contiguous()
+                    for n in ("q.norm", "k.norm", "r1", "r2", "talk", "sink"):
+                        L.w[n] = f32(x + n)
+                L.w["o"] = t(x + "o").detach()
+                f = spec.get("mlp")
+                if f:
+                    L.ff = dict(ff=f["ff"], norm=f32(p + "norm2"), down=t(p + "mlp.down").detach(),
+                                gu=torch.cat([t(p + "mlp.gate"), t(p + "mlp.up")], 0).contiguous())
+                if sd:
+                    L.side = dict(gate=t(p + "side.gate").detach(), proj=t(p + "side.proj").detach(),
+                                  norm=f32(p + "side.norm"), col0=i * sd)
+                self.layers.append(L)
+
+    def new_state(self, slots: int, num_blocks: int, block_size: int, device):
+        return DalavikState(self, slots, num_blocks, block_size, device)
+
+    def run_layers(self, st, tokens, seg, observe=None) -> torch.Tensor:
+        return run_dalavik_layers(self, st, tokens, seg, observe)
+
+    def head(self, x: torch.Tensor) -> torch.Tensor:
+        h = group_rms_norm(x, self.final, self.cfg.norm_groups, self.cfg.rms_norm_eps, self.dtype)
+        return F.linear(h, self.lm_head)
+
+
+class DalavikState:
+    """Paged caches of a Dalavik model: one row [latent | rotated key part] per token for every
+    latent-attention layer that projects its own (a borrowing layer reads the lender's), normed
+    keys and values for every grouped-query layer.  No per-sequence state: ``spare`` only names
+    the slot number graph padding rows carry."""
+
+    def __init__(self, w: DalavikWeights, slots: int, num_blocks: int, block_size: int, device):
+        self.slots = slots
+        self.spare = slots
+        kw = dict(dtype=w.dtype, device=device)
+        self.lat: List[Optional[torch.Tensor]] = []
+        self.k: List[Optional[torch.Tensor]] = []
+        self.v: List[Optional[torch.Tensor]] = []
+        for i, L in enumerate(w.layers):
+            m = L.m
+            own = L.kind == "latent_attention" and L.kv_layer == i
+            self.lat.append(torch.zeros(num_blocks, block_size, m["kv_rank"] + m["rot_dim"], **kw)
+                            if own else None)
+            att = L.kind == "attention"
+            self.k.append(torch.zeros(num_blocks, block_size, m["kv_heads"], m["dim"], **kw)
+                          if att else None)
+            self.v.append(torch.zeros(num_blocks, block_size, m["kv_heads"], m["vdim"], **kw)
+                          if att else None)
+
+
+def run_dalavik_layers(w: DalavikWeights, st: DalavikState, tokens: torch.Tensor, seg: SegBatch,
+                       observe=None) -> torch.Tensor:
+    """The step function: token ids [T] + their segments -> the fp32 residual stream [T, W]
+    after the last layer; the caches in ``st`` take the step's rows."""
+    cfg = w.cfg
+    dt = w.dtype
+    eps, groups = cfg.rms_norm_eps, cfg.norm_groups
+    T = tokens.shape[0]
+    x = F.embedding(tokens, w.embed).float()
+    cast = dt if dt != torch.float32 else None
+    xb = x.to(dt) if cast is not None else x
+    for i, L in enumerate(w.layers):
+        m = L.m
+        if L.kind == "latent_attention":
+            H, D, Dr, Dv, R, Q = (m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"],
+                                  m["q_rank"])
+            z = F.linear(xb, L.w["down"])
+            if L.kv_layer == i:
+                latent_write(z[:, Q:], L.w["dkv_norm"], L.w["inv_freq"], seg.positions,
+                             seg.cache_slots, st.lat[i], R, m["rot"]["dims"], eps)
+            cache = st.lat[L.kv_layer]
+            q = F.linear(group_rms_norm(z[:, :Q], L.w["dq_norm"], 1, eps, dt), L.w["uq"])
+            rotate_interleaved_(q, seg.positions, H, D + Dr, D, m["rot"]["dims"], L.w["inv_freq"])
+            q3 = q.view(T, H, D + Dr)
+            qa = torch.bmm(q3[:, :, :D].transpose(0, 1), L.w["uk"])              # [H, T, R]
+            ol = torch.empty(H, T, R, dtype=dt, device=x.device)
+            row_attention(qa.transpose(0, 1), q3[:, :, D:], cache, cache, R, ol.transpose(0, 1),
+                          seg, H, 1, float(m["scale"]))
+            o = torch.empty(T, H, Dv, dtype=dt, device=x.device)
+            torch.bmm(ol, L.w["uvT"], out=o.transpose(0, 1))
+        else:
+            H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            qkv = F.linear(xb, L.w["qkv"], L.w["qkv_b"])
+            head_norm_write(qkv, L.w["q.norm"], L.w["k.norm"], seg.cache_slots, st.k[i], st.v[i],
+                            H, G, D, Dv, eps)
+            qt = m.get("q_temp")
+            o = torch.empty(T, H, Dv, dtype=dt, device=x.device)
+            row_attention(qkv[:, :H * D].view(T, H, D), None, st.k[i], st.v[i], Dv, o, seg, H, G,
+                          float(m["scale"]), float(m.get("softcap") or 0.0),
+                          (float(qt["coef"]), int(qt["every"])) if qt else None,
+                          L.w["r1"], L.w["r2"], L.w["talk"], L.w["sink"])
+        y = F.linear(o.view(T, H * Dv), L.w["o"])
+        x, xc = group_rms_residual(x, y, L.norm1, groups, eps, cast)
+        xb = xc if cast is not None else x
+        f = L.ff
+        if f is not None:
+            y = F.linear(gated_act(F.linear(xb, f["gu"]), None, 0, 0, f["ff"], "relu"), f["down"])
+            x, xc = group_rms_residual(x, y, f["norm"], groups, eps, cast)
+            xb = xc if cast is not None else x
+        sd = L.side
+        if sd is not None:
+            g = gated_token_slice(F.linear(xb, sd["gate"]), w.side_embed, tokens, sd["col0"])
+            x, xc = group_rms_residual(x, F.linear(g, sd["proj"]), sd["norm"], 1, eps, cast)
+            xb = xc if cast is not None else x
+        if observe is not None:
+            observe(i, x)
+    return x
+
+
+WEIGHTS = {"gedatar": HybridWeights, "dalavik": DalavikWeights}
+
+
 class HybridRunner(ModelRunner):
     """ModelRunner for hybrid stacks: the same step interface (execute / decode / sample, the
     hipGraph decode buckets), its own weights, caches and step function."""
@@ -223,7 +441,7 @@ class HybridRunner(ModelRunner):
         self.tp_group, self.tp, self.car, self.lora = None, 1, None, None
         self.max_blocks = (max_model_len + block_size - 1) // block_size
         self.kv_dtype = weights.dtype
-        self.state = HybridState(weights, state_slots, num_blocks, block_size, device)
+        self.state = weights.new_state(state_slots, num_blocks, block_size, device)
         self.use_graphs = use_graphs and device.type == "cuda"
         self.graph_buckets = [b for b in (1, 2, 4, 8, 16, 32, 64, 96, 128, 160, 192, 224, 256)
                               if b <= max(1, max_graph_batch)]
@@ -237,11 +455,11 @@ class HybridRunner(ModelRunner):
             if rows.numel() == 0:
                 return torch.empty(0, self.cfg.vocab_size, device=x.device, dtype=self.w.dtype)
             x = x[rows]
-        return F.linear(dyt(x, self.w.final, self.w.dtype), self.w.lm_head)
+        return self.w.head(x)
 
     @torch.no_grad()
     def execute(self, inp: StepInput) -> torch.Tensor:
-        x = run_layers(self.w, self.state, inp.tokens, inp.seg, self.observe)
+        x = self.w.run_layers(self.state, inp.tokens, inp.seg, self.observe)
         if inp.extra_rows is not None and inp.extra_rows.numel():
             self.extra_logits = self._logits_rows(x, inp.extra_rows)
         return self._logits_rows(x, inp.sample_rows)
@@ -250,8 +468,8 @@ class HybridRunner(ModelRunner):
 
     # ---- decode: one row per sequence (graph hooks of ModelRunner.decode) --------------------
     def _decode_input(self, inp: StepInput) -> torch.Tensor:
-        return self._logits_rows(run_layers(self.w, self.state, inp.tokens, inp.seg,
-                                            self.observe), None)
+        return self._logits_rows(self.w.run_layers(self.state, inp.tokens, inp.seg,
+                                                   self.observe), None)
 
     def _static_inputs(self, bucket: int) -> dict:
         dev = self.device
@@ -279,18 +497,17 @@ class HybridRunner(ModelRunner):
             sg.cache_slots[N:].fill_(-1)
 
     def _decode_static(self, st: dict) -> torch.Tensor:
-        return self._logits_rows(run_layers(self.w, self.state, st["tokens"], st["seg"]), None)
+        return self._logits_rows(self.w.run_layers(self.state, st["tokens"], st["seg"]), None)
 
 
 @torch.no_grad()
 def forward_fresh(model, input_ids: torch.Tensor, block_size: int = 16) -> torch.Tensor:
-    """Logits [B, S, V] of whole sequences on a private, fresh cache (GedatarForCausalLM.forward)."""
+    """Logits [B, S, V] of whole sequences on a private, fresh cache (the models' ``forward``)."""
     B, S = input_ids.shape
     dev = input_ids.device
-    w = HybridWeights(model)
+    w = WEIGHTS[model.config.arch](model)
     nb = B * ((S + block_size - 1) // block_size)
-    st = HybridState(w, B, nb, block_size, dev)
+    st = w.new_state(B, nb, block_size, dev)
     seg = whole_sequences([S] * B, dev, block_size=block_size)
-    x = run_layers(w, st, input_ids.reshape(-1), seg)
-    y = F.linear(dyt(x, w.final, w.dtype), w.lm_head)
-    return y.view(B, S, -1)
+    x = w.run_layers(st, input_ids.reshape(-1), seg)
+    return w.head(x).view(B, S, -1)
