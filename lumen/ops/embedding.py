@@ -35,13 +35,13 @@ def gated_token_slice(z: torch.Tensor, table: torch.Tensor, tokens: torch.Tensor
     one pass; HIP ``csrc/seqmix/rms_group.hip``)."""
     from ._seqmix import DT, call, use_seqmix
 
+    T, dim = z.shape
+    if col0 < 0 or col0 + dim > table.shape[1]:
+        raise ValueError(f"columns [{col0}, {col0 + dim}) outside a table of {table.shape[1]}")
     if not use_seqmix(z):
         return gated_token_slice_ref(z, table, tokens, col0)
     assert z.stride(1) == 1 and table.stride(1) == 1 and table.dtype == z.dtype
     assert tokens.dtype == torch.int64 and tokens.is_contiguous()
-    T, dim = z.shape
-    if col0 < 0 or col0 + dim > table.shape[1]:
-        raise ValueError(f"columns [{col0}, {col0 + dim}) outside a table of {table.shape[1]}")
     out = torch.empty(T, dim, dtype=z.dtype, device=z.device)
     call("sm_gate_rows", DT[z.dtype], z, z.stride(0), table, table.stride(0), tokens, col0, dim,
          out, T)
