@@ -491,9 +491,10 @@ def main():
                          "region plus a fixed 8192^3 GEMM and a 4 GiB HBM read")
     ap.add_argument("--no_box", dest="box", action="store_false")
     ap.add_argument("--hybrid", action="store_true",
-                    help="instead of the default workload: prefill / decode throughput of the "
-                         "hybrid design (Gedatar) beside Llama at equal size, one GPU "
-                         "(lumen/bench/hybrid_bench.py)")
+                    help="instead of the default workload: prefill / decode throughput of a "
+                         "per-layer-mixer design (--hybrid_family) beside Llama at equal size, "
+                         "one GPU (lumen/bench/hybrid_bench.py)")
+    ap.add_argument("--hybrid_family", default="gedatar", choices=["gedatar", "dalavik"])
     ap.add_argument("--hybrid_widths", default="2048,4096")
     ap.add_argument("--hybrid_batch", default="8,64", help="sequences per step (comma list)")
     ap.add_argument("--hybrid_prompt", type=int, default=512)

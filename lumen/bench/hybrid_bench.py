@@ -1,7 +1,8 @@
-"""Prefill / decode throughput of the hybrid design (Gedatar) beside Llama at equal size.
+"""Prefill / decode throughput of a per-layer-mixer design (Gedatar, Dalavik) beside Llama at
+equal size.
 
-``python bench.py --hybrid`` (one GPU).  Both models get random weights of layer shapes that
-resemble real models (width 2048 / 4096, head size 128 / 64, FFN 2.75 x width, vocab 32000), the
+``python bench.py --hybrid [--hybrid_family dalavik]`` (one GPU).  Both models get random
+weights of layer shapes that resemble real models (width 2048 / 4096, head size 128 / 64, FFN 2.75 x width, vocab 32000), the
 same depth, and run the same forced-token workload through the serving engine
 (``lumen.serve.trace.TraceReplay``: the engine's input builder, block manager, state slots,
 runner, hipGraph decode):
@@ -40,6 +41,36 @@ def gedatar_config(width: int, depth_groups: int = 1):
                        intermediate_size=0, num_attention_heads=0, num_key_value_heads=0,
                        max_position_embeddings=1 << 20, eos_token_id=-1,
                        name=f"gedatar-w{W}", layer_specs=layers)
+
+
+def dalavik_config(width: int, depth_groups: int = 1):
+    """Latent attention at the published shapes of compressed-KV models (heads of 128 + 64
+    rotated, latent 512, query latent 3/4 of the width), one grouped-query layer with every score
+    shaping on, one latent layer that borrows a cache; FFN 2.75 x width; token side input 128."""
+    from ..models.config import ModelConfig
+
+    W = width
+    ff = {"kind": "dense", "ff": int(2.75 * W)}
+    H = W // 128
+
+    def lat(src=None):
+        m = {"heads": H, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512,
+             "q_rank": 3 * W // 4, "scale": 192 ** -0.5, "rot": {"base": 10000.0, "dims": 64}}
+        if src is not None:
+            m["kv_from"] = src
+        return {"type": "latent_attention", "mixer": m, "mlp": ff}
+
+    att = {"type": "attention", "mlp": ff,
+           "mixer": {"heads": H, "kv_heads": max(1, W // 512), "dim": 128, "vdim": 128,
+                     "scale": 128 ** -0.5, "softcap": 30.0, "q_temp": {"coef": 0.1, "every": 1024}}}
+    layers = []
+    for g in range(depth_groups):
+        layers += [lat(), lat(), att, lat(4 * g + 1)]
+    return ModelConfig(arch="dalavik", vocab_size=32000, hidden_size=W,
+                       num_hidden_layers=len(layers), rms_norm_eps=1e-6, norm_groups=4,
+                       token_side_dim=128, intermediate_size=0, num_attention_heads=0,
+                       num_key_value_heads=0, max_position_embeddings=1 << 20, eos_token_id=-1,
+                       tie_word_embeddings=True, name=f"dalavik-w{W}", layer_specs=layers)
 
 
 def llama_config(width: int, layers: int):
@@ -115,8 +146,10 @@ def run_hybrid_bench(args) -> list:
 
     assert native() is not None, native_error()
     rows = []
+    family = getattr(args, "hybrid_family", "gedatar")
+    make = {"gedatar": gedatar_config, "dalavik": dalavik_config}[family]
     for width in [int(w) for w in str(args.hybrid_widths).split(",")]:
-        gcfg = gedatar_config(width)
+        gcfg = make(width)
         for cfg in (gcfg, llama_config(width, gcfg.num_hidden_layers)):
             for batch in [int(b) for b in str(args.hybrid_batch).split(",")]:
                 r = run_one(cfg, batch, args.hybrid_prompt, args.hybrid_decode_steps, 3, dev)
@@ -126,12 +159,13 @@ def run_hybrid_bench(args) -> list:
     by = {(r["width"], r["batch"], r["model"].split("-")[0]): r for r in rows}
     summ = []
     for (w, b, kind), r in by.items():
-        if kind != "gedatar":
+        if kind != family:
             continue
         ll = by[(w, b, "llama")]
         summ.append({"width": w, "batch": b,
                      "prefill_vs_llama": round(r["prefill_tok_s"] / ll["prefill_tok_s"], 3),
                      "decode_vs_llama": round(r["decode_tok_s"] / ll["decode_tok_s"], 3)})
-    print(json.dumps({"metric": "hybrid_vs_llama_tokens_per_s", "dtype": "bf16",
+    metric = "hybrid" if family == "gedatar" else family
+    print(json.dumps({"metric": f"{metric}_vs_llama_tokens_per_s", "dtype": "bf16",
                       "data": "synthetic", "rows": summ}), flush=True)
     return rows

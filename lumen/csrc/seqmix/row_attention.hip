@@ -22,7 +22,9 @@
 //
 // One workgroup of four waves per (row, block of HB heads): a row is a row, whether it belongs
 // to a prompt's portion or is a decoded token, so its result cannot depend on how a step was
-// cut.  Keys are visited 64 at a time, lane = key.  The waves share the heads of the block out
+// cut.  When a step has few rows (decoding), a row's 64-key tiles are dealt out to `nsplit`
+// workgroups whose partial (max, sum, accumulator) a small second kernel merges, so that the chip
+// is filled whatever the batch.  Keys are visited 64 at a time, lane = key.  The waves share the heads of the block out
 // among themselves (head w, w + 4, ...): a wave scores its heads against the tile, the scores of
 // all heads meet in LDS (double-buffered, one barrier per tile) where the head mixing reads
 // them, then every wave runs the online softmax and the value pass of its own heads; lanes own
@@ -137,6 +139,7 @@ struct RowAttnArgs {
   int H, G, HB, bs;
   float scale, softcap, tcoef; int tevery;
   const float *r1, *r2, *talk, *sink;
+  int nsplit; float* ws_ml; float* ws_o;     // key splits: partial (max, sum) and accumulators
 };
 
 template <typename T, int HPW>
@@ -173,7 +176,7 @@ row_attn_kernel(const RowAttnArgs<T> a) {
 #pragma unroll
   for (int i = 0; i < HPW; ++i) {
     const int hl = w + kWaves * i;
-    const bool sk = a.sink != nullptr && hl < nh;
+    const bool sk = a.sink != nullptr && hl < nh && blockIdx.z == 0;
     m[i] = sk ? a.sink[h0 + hl] : -INFINITY;     // the sink: a key of score sink_h, no value
     l[i] = sk ? 1.f : 0.f;
 #pragma unroll
@@ -186,7 +189,7 @@ row_attn_kernel(const RowAttnArgs<T> a) {
   __syncthreads();
 
   int buf = 0;
-  for (int j0 = 0; j0 <= pos; j0 += 64, buf ^= 1) {
+  for (int j0 = 64 * blockIdx.z; j0 <= pos; j0 += 64 * a.nsplit, buf ^= 1) {
     const int j = j0 + lane;
     const bool valid = j <= pos;
     const int rb = valid ? tbl[j / a.bs] * a.bs + j % a.bs : 0;
@@ -296,10 +299,48 @@ row_attn_kernel(const RowAttnArgs<T> a) {
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     }
-    const float inv = 1.f / l[i];
-    T* op = a.out + (long long)t * a.our + (long long)h * a.ouh;
-    for (int d = lane; d < a.Dv; d += 64) op[d] = from_f32<T>(so[d] * inv);
+    if (a.nsplit == 1) {
+      const float inv = 1.f / l[i];
+      T* op = a.out + (long long)t * a.our + (long long)h * a.ouh;
+      for (int d = lane; d < a.Dv; d += 64) op[d] = from_f32<T>(so[d] * inv);
+    } else {
+      // this split's running state, un-normalised; row_attn_combine merges the splits
+      const long long slot = ((long long)t * a.H + h) * a.nsplit + blockIdx.z;
+      if (lane == 0) {
+        a.ws_ml[2 * slot] = m[i];
+        a.ws_ml[2 * slot + 1] = l[i];
+      }
+      for (int d = lane; d < a.Dv; d += 64) a.ws_o[slot * a.Dv + d] = so[d];
+    }
     __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// out[t, h] = sum_s acc_s exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s: the splits of a
+// row's keys merged; a split that saw no key has (m, l) = (-inf, 0) and drops out
+template <typename T>
+__global__ void __launch_bounds__(64)
+row_attn_combine_kernel(const float* __restrict__ ws_ml, const float* __restrict__ ws_o,
+                        T* __restrict__ out, long long our, long long ouh, int H, int Dv,
+                        int nsplit) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const long long base = ((long long)t * H + h) * nsplit;
+  float M = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, ws_ml[2 * (base + s)]);
+  float L = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float ms = ws_ml[2 * (base + s)];
+    if (ms != -INFINITY) L += ws_ml[2 * (base + s) + 1] * expf(ms - M);
+  }
+  const float inv = 1.f / L;
+  T* op = out + (long long)t * our + (long long)h * ouh;
+  for (int d = lane; d < Dv; d += 64) {
+    float o = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float ms = ws_ml[2 * (base + s)];
+      if (ms != -INFINITY) o += ws_o[(base + s) * Dv + d] * expf(ms - M);
+    }
+    op[d] = from_f32<T>(o * inv);
   }
 }
 
@@ -312,13 +353,16 @@ template <typename T>
 hipError_t launch_row_attn(const RowAttnArgs<T>& a, int Tn, hipStream_t st) {
   const int Dk = a.D1 + a.D2;
   const size_t lds = row_attn_lds(a.HB, Dk);
-  const dim3 grid(Tn, (a.H + a.HB - 1) / a.HB);
+  const dim3 grid(Tn, (a.H + a.HB - 1) / a.HB, a.nsplit);
   const int hpw = (a.HB + kWaves - 1) / kWaves;
   if (hpw <= 1) row_attn_kernel<T, 1><<<grid, 64 * kWaves, lds, st>>>(a);
   else if (hpw <= 2) row_attn_kernel<T, 2><<<grid, 64 * kWaves, lds, st>>>(a);
   else if (hpw <= 4) row_attn_kernel<T, 4><<<grid, 64 * kWaves, lds, st>>>(a);
   else if (hpw <= 8) row_attn_kernel<T, 8><<<grid, 64 * kWaves, lds, st>>>(a);
   else return hipErrorInvalidValue;
+  if (a.nsplit > 1)
+    row_attn_combine_kernel<T><<<dim3(Tn, a.H), 64, 0, st>>>(a.ws_ml, a.ws_o, a.out, a.our, a.ouh,
+                                                             a.H, a.Dv, a.nsplit);
   return hipGetLastError();
 }
 
@@ -375,8 +419,9 @@ hipError_t sm_row_attn(int dt, const void* q1, long long q1r, long long q1h, int
                        const int* row_seg, const int* positions, int T, int H, int G, int HB,
                        int bs, float scale, float softcap, float tcoef, int tevery,
                        const float* r1, const float* r2, const float* talk, const float* sink,
-                       hipStream_t st) {
+                       int nsplit, float* ws_ml, float* ws_o, hipStream_t st) {
   if (T == 0) return hipSuccess;
+  if (nsplit < 1 || nsplit > 65535 || (nsplit > 1 && (!ws_ml || !ws_o))) return hipErrorInvalidValue;
   if (H % G != 0 || HB < 1 || HB > 8 * kWaves || Dv > kMaxDv || (talk && HB < H) ||
       (D2 > 0 && q2 == nullptr) || row_attn_lds(HB, D1 + D2) > 65536)
     return hipErrorInvalidValue;
@@ -385,7 +430,7 @@ hipError_t sm_row_attn(int dt, const void* q1, long long q1r, long long q1h, int
     RowAttnArgs<TT> a{(const TT*)q1, q1r, q1h, D1, (const TT*)q2, q2r, q2h, D2,               \
                       (const TT*)kc, krow, (const TT*)vc, vrow, Dv, (TT*)out, our, ouh,       \
                       tables, maxb, row_seg, positions, H, G, HB, bs, scale, softcap, tcoef,  \
-                      tevery, r1, r2, talk, sink};                                            \
+                      tevery, r1, r2, talk, sink, nsplit, ws_ml, ws_o};                                         \
     return launch_row_attn<TT>(a, T, st);                                                     \
   }
   SM_DISPATCH(dt, CALL)

@@ -38,7 +38,7 @@ SIGNATURES = {
     "sm_rotate_heads": "iplliiippi",
     "sm_latent_write": "iplpppppiiiif",
     "sm_head_norm_write": "iplpppppiiiiif",
-    "sm_row_attn": "i" "plli" "plli" "pl" "pli" "pll" "pi" "pp" "iiiii" "fffi" "pppp",
+    "sm_row_attn": "i" "plli" "plli" "pl" "pli" "pll" "pi" "pp" "iiiii" "fffi" "pppp" "ipp",
 }
 
 

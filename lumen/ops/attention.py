@@ -751,9 +751,21 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
         assert f is None or (f.dtype == torch.float32 and f.is_contiguous())
     HB = _heads_per_block(H, Dk, talk is not None)
     coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp is not None else (0.0, 0)
+    # few rows (decoding): deal a row's 64-key tiles out to several workgroups so that ~2 per CU
+    # run; the count depends on the step's size only, never on device data (graph capture)
+    tiles = (seg.tables.shape[1] * kcache.shape[1] + 63) // 64
+    while talk is None and HB > 4 and T * ((H + HB - 1) // HB) * tiles < 512:
+        HB //= 2                       # fewer heads per workgroup: more workgroups
+    blocks = T * ((H + HB - 1) // HB)
+    nsplit = max(1, min(tiles, 32, 512 // max(blocks, 1)))
+    ws_ml = ws_o = None
+    if nsplit > 1:
+        ws_ml = torch.empty(T * H * nsplit * 2, dtype=torch.float32, device=q1.device)
+        ws_o = torch.empty(T * H * nsplit * Dv, dtype=torch.float32, device=q1.device)
     call("sm_row_attn", DT[q1.dtype], q1, q1.stride(0), q1.stride(1), D1,
          q2, q2.stride(0) if q2 is not None else 0, q2.stride(1) if q2 is not None else 0, D2,
          kcache, krow, vcache, vrow, Dv, out, out.stride(0), out.stride(1),
          seg.tables, seg.tables.shape[1], seg.row_seg, seg.positions, T, H, G, HB,
-         kcache.shape[1], scale, float(softcap or 0.0), coef, every, r1, r2, talk, sink)
+         kcache.shape[1], scale, float(softcap or 0.0), coef, every, r1, r2, talk, sink,
+         nsplit, ws_ml, ws_o)
     return out
