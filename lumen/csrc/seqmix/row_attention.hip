@@ -38,6 +38,32 @@ namespace {
 
 constexpr int kWaves = 4;
 constexpr int kMaxDv = 512;
+constexpr int kQPad = 8;      // padding of the 16-bit query rows in LDS (bank spread)
+
+// v_mfma_f32_16x16x32: lane l holds A[m = l & 15][k = 8 (l >> 4) + 0..7] and
+// B[k = 8 (l >> 4) + 0..7][n = l & 15]; the accumulator register i is C[4 (l >> 4) + i][l & 15]
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8r __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8r __attribute__((ext_vector_type(8)));
+template <typename T> struct Mma16 { static constexpr bool ok = false; };
+template <> struct Mma16<bf16> {
+  static constexpr bool ok = true;
+  static __device__ __forceinline__ f32x4v run(uint4 a, uint4 b, f32x4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8r, a),
+                                                   __builtin_bit_cast(bf16x8r, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma16<fp16> {
+  static constexpr bool ok = true;
+  static __device__ __forceinline__ f32x4v run(uint4 a, uint4 b, f32x4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8r, a),
+                                                  __builtin_bit_cast(f16x8r, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma16<float> {
+  static constexpr bool ok = false;
+  static __device__ __forceinline__ f32x4v run(uint4, uint4, f32x4v c) { return c; }
+};
 
 template <typename T>
 __global__ void rotate_heads_kernel(T* __restrict__ x, long long ldr, long long ldh, int heads,
@@ -142,7 +168,13 @@ struct RowAttnArgs {
   int nsplit; float* ws_ml; float* ws_o;     // key splits: partial (max, sum) and accumulators
 };
 
-template <typename T, int HPW>
+// MMA (16-bit dtypes, one key/value head, at most 16 heads per workgroup, key size a multiple of
+// 8): the tile's scores come from the matrix cores as S^T = K Q^T -- wave w takes keys
+// 16 w .. 16 w + 15 of the tile against ALL heads of the block; a lane loads 16 bytes of ITS key's
+// row per step (the contracted dimension is contiguous in both operands, so nothing is
+// transposed), the queries wait in LDS in 16 bits exactly as projected, and the fp32 products land
+// in the same LDS score buffer the vector path fills.
+template <typename T, int HPW, bool MMA>
 __global__ void __launch_bounds__(64 * kWaves)
 row_attn_kernel(const RowAttnArgs<T> a) {
   extern __shared__ float smem[];
@@ -155,17 +187,31 @@ row_attn_kernel(const RowAttnArgs<T> a) {
   const int hpg = a.H / a.G;
   // LDS: queries [HB][Dk] | scores [2][HB][64] | weights [HB][64] | reduction [4][kMaxDv] |
   // cache rows of the tile's keys [2][64]
+  const int Dkp = (Dk + 31) / 32 * 32;          // MMA: rows padded with zeros to the 32-wide step
   float* s_q = smem;
-  float* s_sc = s_q + (long long)a.HB * Dk;
+  T* s_qb = reinterpret_cast<T*>(smem);
+  float* s_sc = s_q + (MMA ? (16 * (Dkp + kQPad) * (int)sizeof(T) + 3) / 4 : a.HB * Dk);
   float* s_p = s_sc + 2 * a.HB * 64;
   float* s_o = s_p + a.HB * 64;
   int* s_rb = reinterpret_cast<int*>(s_o + kWaves * kMaxDv);
 
-  for (int i = threadIdx.x; i < nh * Dk; i += 64 * kWaves) {
-    const int hl = i / Dk, d = i % Dk;
-    const int h = h0 + hl;
-    s_q[i] = d < a.D1 ? to_f32(a.q1[(long long)t * a.q1r + (long long)h * a.q1h + d])
-                      : to_f32(a.q2[(long long)t * a.q2r + (long long)h * a.q2h + (d - a.D1)]);
+  if (MMA) {
+    for (int i = threadIdx.x; i < 16 * Dkp; i += 64 * kWaves) {
+      const int hl = i / Dkp, d = i % Dkp;
+      const int h = h0 + hl;
+      T v = from_f32<T>(0.f);
+      if (hl < nh && d < Dk)
+        v = d < a.D1 ? a.q1[(long long)t * a.q1r + (long long)h * a.q1h + d]
+                     : a.q2[(long long)t * a.q2r + (long long)h * a.q2h + (d - a.D1)];
+      s_qb[hl * (Dkp + kQPad) + d] = v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < nh * Dk; i += 64 * kWaves) {
+      const int hl = i / Dk, d = i % Dk;
+      const int h = h0 + hl;
+      s_q[i] = d < a.D1 ? to_f32(a.q1[(long long)t * a.q1r + (long long)h * a.q1h + d])
+                        : to_f32(a.q2[(long long)t * a.q2r + (long long)h * a.q2h + (d - a.D1)]);
+    }
   }
   float temp = 1.f;
   if (a.tevery > 0 && a.tcoef != 0.f)
@@ -195,32 +241,62 @@ row_attn_kernel(const RowAttnArgs<T> a) {
     const int rb = valid ? tbl[j / a.bs] * a.bs + j % a.bs : 0;
     if (w == 0) s_rb[buf * 64 + lane] = rb;
     const float dist = (float)(pos - j);
-#pragma unroll
-    for (int i = 0; i < HPW; ++i) {
-      const int hl = w + kWaves * i;
-      if (hl >= nh) break;
-      const int h = h0 + hl;
-      float dot = 0.f;
-      if (valid) {
-        const T* kp = a.kc + (long long)rb * a.krow + (long long)(h / hpg) * Dk;
-        const float* qh = s_q + hl * Dk;
-        if (kvec) {
-          for (int d = 0; d < Dk; d += 8) {
-            float kv[8];
-            load8<T>(kp + d, kv);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) dot += qh[d + e] * kv[e];
-          }
-        } else {
-          for (int d = 0; d < Dk; ++d) dot += qh[d] * to_f32(kp[d]);
+    if (MMA) {
+      const int key = lane & 15, kg = lane >> 4;
+      const int jk = j0 + 16 * w + key;
+      const long long rbk = jk <= pos ? (long long)tbl[jk / a.bs] * a.bs + jk % a.bs : 0;
+      const T* kp = a.kc + rbk * a.krow;
+      const T* qp = s_qb + key * (Dkp + kQPad);          // as B operand: the lane's head = lane & 15
+      f32x4v c = {0.f, 0.f, 0.f, 0.f};
+      if (16 * w <= pos - j0) {                          // the wave's 16 keys hold a visible one
+        for (int d0 = 0; d0 < Dkp; d0 += 32) {
+          const int d = d0 + 8 * kg;
+          uint4 av = make_uint4(0u, 0u, 0u, 0u);
+          if (d < Dk) av = *reinterpret_cast<const uint4*>(kp + d);
+          const uint4 bv = *reinterpret_cast<const uint4*>(qp + d);
+          c = Mma16<T>::run(av, bv, c);
         }
       }
-      float s = dot * qscale;
-      if (a.softcap > 0.f) s = a.softcap * tanhf(s / a.softcap);
-      if (a.r1 != nullptr) s -= a.r1[h] * logf(1.f + a.r2[h] * dist);
-      s = valid ? s : 0.f;
-      sreg[i] = s;
-      s_sc[(buf * a.HB + hl) * 64 + lane] = s;
+      const int hl = lane & 15;                          // c[i] = S^T[key 4 kg + i][head hl]
+      if (hl < nh) {
+        const int h = h0 + hl;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int kk = 16 * w + 4 * kg + i;
+          float sv = c[i] * qscale;
+          if (a.softcap > 0.f) sv = a.softcap * tanhf(sv / a.softcap);
+          if (a.r1 != nullptr) sv -= a.r1[h] * logf(1.f + a.r2[h] * (float)(pos - j0 - kk));
+          s_sc[(buf * a.HB + hl) * 64 + kk] = j0 + kk <= pos ? sv : 0.f;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < HPW; ++i) {
+        const int hl = w + kWaves * i;
+        if (hl >= nh) break;
+        const int h = h0 + hl;
+        float dot = 0.f;
+        if (valid) {
+          const T* kp = a.kc + (long long)rb * a.krow + (long long)(h / hpg) * Dk;
+          const float* qh = s_q + hl * Dk;
+          if (kvec) {
+            for (int d = 0; d < Dk; d += 8) {
+              float kv[8];
+              load8<T>(kp + d, kv);
+#pragma unroll
+              for (int e = 0; e < 8; ++e) dot += qh[d + e] * kv[e];
+            }
+          } else {
+            for (int d = 0; d < Dk; ++d) dot += qh[d] * to_f32(kp[d]);
+          }
+        }
+        float sv = dot * qscale;
+        if (a.softcap > 0.f) sv = a.softcap * tanhf(sv / a.softcap);
+        if (a.r1 != nullptr) sv -= a.r1[h] * logf(1.f + a.r2[h] * dist);
+        sv = valid ? sv : 0.f;
+        sreg[i] = sv;
+        s_sc[(buf * a.HB + hl) * 64 + lane] = sv;
+      }
     }
     __syncthreads();
     const int nk = min(64, pos - j0 + 1);
@@ -229,7 +305,7 @@ row_attn_kernel(const RowAttnArgs<T> a) {
       const int hl = w + kWaves * i;
       if (hl >= nh) break;
       const int h = h0 + hl;
-      float s = sreg[i];
+      float s = MMA ? s_sc[(buf * a.HB + hl) * 64 + lane] : sreg[i];
       if (a.talk != nullptr) {
         s = 0.f;
         for (int g = 0; g < nh; ++g) s += a.talk[h * a.H + h0 + g] * s_sc[(buf * a.HB + g) * 64 + lane];
@@ -243,32 +319,56 @@ row_attn_kernel(const RowAttnArgs<T> a) {
       s_p[hl * 64 + lane] = p;
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[i][e] *= corr;
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      const long long voff = (long long)(h / hpg) * a.Dv;
-      if (vvec) {
-        if (grp < kpi) {
-          for (int jj = grp; jj < nk; jj += kpi) {
-            const float pj = s_p[hl * 64 + jj];
-            float vv[8];
-            load8<T>(a.vc + (long long)s_rb[buf * 64 + jj] * a.vrow + voff + 8 * part, vv);
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    if (vvec && a.G == 1) {
+      // one key/value head: a value row is loaded once for all heads of the wave
+      if (grp < kpi) {
+        for (int jj = grp; jj < nk; jj += kpi) {
+          float vv[8];
+          load8<T>(a.vc + (long long)s_rb[buf * 64 + jj] * a.vrow + 8 * part, vv);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[i][e] += pj * vv[e];
-          }
-        }
-      } else {
-        for (int jj = 0; jj < nk; ++jj) {
-          const float pj = s_p[hl * 64 + jj];
-          const T* vp = a.vc + (long long)s_rb[buf * 64 + jj] * a.vrow + voff;
+          for (int i = 0; i < HPW; ++i) {
+            const int hl = w + kWaves * i;
+            if (hl < nh) {
+              const float pj = s_p[hl * 64 + jj];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const int d = lane + 64 * e;
-            if (d < a.Dv) acc[i][e] += pj * to_f32(vp[d]);
+              for (int e = 0; e < 8; ++e) acc[i][e] += pj * vv[e];
+            }
           }
         }
       }
-      __builtin_amdgcn_wave_barrier();
+    } else {
+#pragma unroll
+      for (int i = 0; i < HPW; ++i) {
+        const int hl = w + kWaves * i;
+        if (hl >= nh) break;
+        const long long voff = (long long)((h0 + hl) / hpg) * a.Dv;
+        if (vvec) {
+          if (grp < kpi) {
+            for (int jj = grp; jj < nk; jj += kpi) {
+              const float pj = s_p[hl * 64 + jj];
+              float vv[8];
+              load8<T>(a.vc + (long long)s_rb[buf * 64 + jj] * a.vrow + voff + 8 * part, vv);
+#pragma unroll
+              for (int e = 0; e < 8; ++e) acc[i][e] += pj * vv[e];
+            }
+          }
+        } else {
+          for (int jj = 0; jj < nk; ++jj) {
+            const float pj = s_p[hl * 64 + jj];
+            const T* vp = a.vc + (long long)s_rb[buf * 64 + jj] * a.vrow + voff;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const int d = lane + 64 * e;
+              if (d < a.Dv) acc[i][e] += pj * to_f32(vp[d]);
+            }
+          }
+        }
+      }
     }
+    __builtin_amdgcn_wave_barrier();
   }
 
   float* so = s_o + w * kMaxDv;
@@ -319,50 +419,67 @@ row_attn_kernel(const RowAttnArgs<T> a) {
 // out[t, h] = sum_s acc_s exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s: the splits of a
 // row's keys merged; a split that saw no key has (m, l) = (-inf, 0) and drops out
 template <typename T>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
 row_attn_combine_kernel(const float* __restrict__ ws_ml, const float* __restrict__ ws_o,
                         T* __restrict__ out, long long our, long long ouh, int H, int Dv,
                         int nsplit) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63;
   const long long base = ((long long)t * H + h) * nsplit;
-  float M = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, ws_ml[2 * (base + s)]);
-  float L = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float ms = ws_ml[2 * (base + s)];
-    if (ms != -INFINITY) L += ws_ml[2 * (base + s) + 1] * expf(ms - M);
+  __shared__ float s_w[64];
+  if (threadIdx.x < 64) {                                // nsplit <= 64: lane s weighs split s
+    const float ms = lane < nsplit ? ws_ml[2 * (base + lane)] : -INFINITY;
+    const float ls = lane < nsplit ? ws_ml[2 * (base + lane) + 1] : 0.f;
+    const float M = wave_max(ms);
+    const float e = ms == -INFINITY ? 0.f : expf(ms - M);
+    const float L = wave_sum(ls * e);
+    s_w[lane] = e / L;
   }
-  const float inv = 1.f / L;
+  __syncthreads();
   T* op = out + (long long)t * our + (long long)h * ouh;
-  for (int d = lane; d < Dv; d += 64) {
+  for (int d = threadIdx.x; d < Dv; d += 256) {
     float o = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-      const float ms = ws_ml[2 * (base + s)];
-      if (ms != -INFINITY) o += ws_o[(base + s) * Dv + d] * expf(ms - M);
-    }
-    op[d] = from_f32<T>(o * inv);
+    for (int s = 0; s < nsplit; ++s) o += ws_o[(base + s) * Dv + d] * s_w[s];
+    op[d] = from_f32<T>(o);
   }
 }
 
-inline size_t row_attn_lds(int HB, int Dk) {
-  return sizeof(float) * ((size_t)HB * Dk + 3 * (size_t)HB * 64 + kWaves * kMaxDv) +
-         sizeof(int) * 2 * 64;
+inline size_t row_attn_lds(int HB, int Dk, bool mma = false, int esz = 2) {
+  const size_t q = mma ? ((size_t)16 * ((Dk + 31) / 32 * 32 + kQPad) * esz + 3) / 4 * 4
+                       : sizeof(float) * (size_t)HB * Dk;
+  return q + sizeof(float) * (3 * (size_t)HB * 64 + kWaves * kMaxDv) + sizeof(int) * 2 * 64;
+}
+
+template <typename T>
+bool row_attn_mma_ok(const RowAttnArgs<T>& a) {
+  const int Dk = a.D1 + a.D2;
+  return Mma16<T>::ok && a.G == 1 && a.HB <= 16 && Dk % 8 == 0 && a.D1 % 8 == 0 &&
+         a.krow % 8 == 0 && ((uintptr_t)a.kc % 16 == 0);
 }
 
 template <typename T>
 hipError_t launch_row_attn(const RowAttnArgs<T>& a, int Tn, hipStream_t st) {
   const int Dk = a.D1 + a.D2;
-  const size_t lds = row_attn_lds(a.HB, Dk);
+  const bool mma = row_attn_mma_ok(a);
+  const size_t lds = row_attn_lds(a.HB, Dk, mma, sizeof(T));
+  if (lds > 65536) return hipErrorInvalidValue;
   const dim3 grid(Tn, (a.H + a.HB - 1) / a.HB, a.nsplit);
   const int hpw = (a.HB + kWaves - 1) / kWaves;
-  if (hpw <= 1) row_attn_kernel<T, 1><<<grid, 64 * kWaves, lds, st>>>(a);
-  else if (hpw <= 2) row_attn_kernel<T, 2><<<grid, 64 * kWaves, lds, st>>>(a);
-  else if (hpw <= 4) row_attn_kernel<T, 4><<<grid, 64 * kWaves, lds, st>>>(a);
-  else if (hpw <= 8) row_attn_kernel<T, 8><<<grid, 64 * kWaves, lds, st>>>(a);
-  else return hipErrorInvalidValue;
+#define LAUNCH(N, M) row_attn_kernel<T, N, M><<<grid, 64 * kWaves, lds, st>>>(a)
+  if (mma) {
+    if (hpw <= 1) LAUNCH(1, true);
+    else if (hpw <= 2) LAUNCH(2, true);
+    else LAUNCH(4, true);
+  } else {
+    if (hpw <= 1) LAUNCH(1, false);
+    else if (hpw <= 2) LAUNCH(2, false);
+    else if (hpw <= 4) LAUNCH(4, false);
+    else if (hpw <= 8) LAUNCH(8, false);
+    else return hipErrorInvalidValue;
+  }
+#undef LAUNCH
   if (a.nsplit > 1)
-    row_attn_combine_kernel<T><<<dim3(Tn, a.H), 64, 0, st>>>(a.ws_ml, a.ws_o, a.out, a.our, a.ouh,
-                                                             a.H, a.Dv, a.nsplit);
+    row_attn_combine_kernel<T><<<dim3(Tn, a.H), 256, 0, st>>>(a.ws_ml, a.ws_o, a.out, a.our, a.ouh,
+                                                              a.H, a.Dv, a.nsplit);
   return hipGetLastError();
 }
 
@@ -410,7 +527,7 @@ hipError_t sm_head_norm_write(int dt, void* qkv, long long ld, const float* wq, 
 }
 
 // LDS bytes a (HB heads, key size Dk) block needs; the caller picks HB so that this fits 64 KB
-int sm_row_attn_lds(int HB, int Dk) { return (int)row_attn_lds(HB, Dk); }
+int sm_row_attn_lds(int HB, int Dk) { return (int)row_attn_lds(HB, Dk, false); }
 
 hipError_t sm_row_attn(int dt, const void* q1, long long q1r, long long q1h, int D1,
                        const void* q2, long long q2r, long long q2h, int D2, const void* kc,
@@ -421,9 +538,9 @@ hipError_t sm_row_attn(int dt, const void* q1, long long q1r, long long q1h, int
                        const float* r1, const float* r2, const float* talk, const float* sink,
                        int nsplit, float* ws_ml, float* ws_o, hipStream_t st) {
   if (T == 0) return hipSuccess;
-  if (nsplit < 1 || nsplit > 65535 || (nsplit > 1 && (!ws_ml || !ws_o))) return hipErrorInvalidValue;
+  if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!ws_ml || !ws_o))) return hipErrorInvalidValue;
   if (H % G != 0 || HB < 1 || HB > 8 * kWaves || Dv > kMaxDv || (talk && HB < H) ||
-      (D2 > 0 && q2 == nullptr) || row_attn_lds(HB, D1 + D2) > 65536)
+      (D2 > 0 && q2 == nullptr))
     return hipErrorInvalidValue;
 #define CALL(TT)                                                                              \
   {                                                                                           \
