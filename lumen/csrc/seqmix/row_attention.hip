@@ -25,7 +25,7 @@
 // cut.  When a step has few rows (decoding), a row's 64-key tiles are dealt out to `nsplit`
 // workgroups whose partial (max, sum, accumulator) a small second kernel merges, so that the chip
 // is filled whatever the batch.  Keys are visited 64 at a time, lane = key.  The waves share the heads of the block out
-// among themselves (head w, w + 4, ...): a wave scores its heads against the tile, the scores of
+// among themselves (consecutive ones each): a wave scores its heads against the tile, the scores of
 // all heads meet in LDS (double-buffered, one barrier per tile) where the head mixing reads
 // them, then every wave runs the online softmax and the value pass of its own heads; lanes own
 // 8 output channels of one key group in the value pass (16-byte loads).  Scores, weights, sums
@@ -168,12 +168,12 @@ struct RowAttnArgs {
   int nsplit; float* ws_ml; float* ws_o;     // key splits: partial (max, sum) and accumulators
 };
 
-// MMA (16-bit dtypes, one key/value head, at most 16 heads per workgroup, key size a multiple of
-// 8): the tile's scores come from the matrix cores as S^T = K Q^T -- wave w takes keys
-// 16 w .. 16 w + 15 of the tile against ALL heads of the block; a lane loads 16 bytes of ITS key's
-// row per step (the contracted dimension is contiguous in both operands, so nothing is
-// transposed), the queries wait in LDS in 16 bits exactly as projected, and the fp32 products land
-// in the same LDS score buffer the vector path fills.
+// MMA (16-bit dtypes, key size and strides multiples of 8): the tile's scores come from the
+// matrix cores as S^T = K Q^T -- wave w takes keys 16 w .. 16 w + 15 of the tile against ALL
+// heads of the block, one chain of products per key/value head the block's heads use and per 16
+// heads; a lane loads 16 bytes of ITS key's row per step (the contracted dimension is contiguous
+// in both operands, so nothing is transposed), the queries wait in LDS in 16 bits exactly as
+// projected, and the fp32 products land in the same LDS score buffer the vector path fills.
 template <typename T, int HPW, bool MMA>
 __global__ void __launch_bounds__(64 * kWaves)
 row_attn_kernel(const RowAttnArgs<T> a) {
@@ -185,25 +185,30 @@ row_attn_kernel(const RowAttnArgs<T> a) {
   const int pos = a.positions[t];
   const int* tbl = a.tables + (long long)a.row_seg[t] * a.maxb;
   const int hpg = a.H / a.G;
-  // LDS: queries [HB][Dk] | scores [2][HB][64] | weights [HB][64] | reduction [4][kMaxDv] |
-  // cache rows of the tile's keys [2][64]
+  // LDS: queries (fp32 [HB][Dk], or 16-bit [16 NB][Dkp + pad]) | scores [2][HB][64] |
+  // weights [HB][64] | reduction [4][kMaxDv] | cache rows of the tile's keys [2][64]
   const int Dkp = (Dk + 31) / 32 * 32;          // MMA: rows padded with zeros to the 32-wide step
+  const int NB = (a.HB + 15) / 16;              // MMA: blocks of 16 heads
   float* s_q = smem;
   T* s_qb = reinterpret_cast<T*>(smem);
-  float* s_sc = s_q + (MMA ? (16 * (Dkp + kQPad) * (int)sizeof(T) + 3) / 4 : a.HB * Dk);
+  float* s_sc = s_q + (MMA ? (16 * NB * (Dkp + kQPad) * (int)sizeof(T) + 3) / 4 : a.HB * Dk);
   float* s_p = s_sc + 2 * a.HB * 64;
   float* s_o = s_p + a.HB * 64;
   int* s_rb = reinterpret_cast<int*>(s_o + kWaves * kMaxDv);
 
   if (MMA) {
-    for (int i = threadIdx.x; i < 16 * Dkp; i += 64 * kWaves) {
-      const int hl = i / Dkp, d = i % Dkp;
+    // 8 elements (16 bytes) per thread; mma_ok guarantees the alignment of both query parts
+    const int cpr = Dkp / 8;
+    for (int c = threadIdx.x; c < 16 * NB * cpr; c += 64 * kWaves) {
+      const int hl = c / cpr, d = (c % cpr) * 8;
       const int h = h0 + hl;
-      T v = from_f32<T>(0.f);
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
       if (hl < nh && d < Dk)
-        v = d < a.D1 ? a.q1[(long long)t * a.q1r + (long long)h * a.q1h + d]
-                     : a.q2[(long long)t * a.q2r + (long long)h * a.q2h + (d - a.D1)];
-      s_qb[hl * (Dkp + kQPad) + d] = v;
+        v = d < a.D1
+                ? *reinterpret_cast<const uint4*>(a.q1 + (long long)t * a.q1r + (long long)h * a.q1h + d)
+                : *reinterpret_cast<const uint4*>(a.q2 + (long long)t * a.q2r + (long long)h * a.q2h +
+                                                  (d - a.D1));
+      *reinterpret_cast<uint4*>(s_qb + hl * (Dkp + kQPad) + d) = v;
     }
   } else {
     for (int i = threadIdx.x; i < nh * Dk; i += 64 * kWaves) {
@@ -218,13 +223,16 @@ row_attn_kernel(const RowAttnArgs<T> a) {
     temp = 1.f + a.tcoef * logf((float)((pos + 1) / a.tevery) + 1.f);
   const float qscale = a.scale * temp;
 
+  // the wave's heads: HPW consecutive ones, so that heads of one key/value head share its rows
+  const int hw0 = w * HPW;
   float m[HPW], l[HPW], acc[HPW][8], sreg[HPW];
 #pragma unroll
   for (int i = 0; i < HPW; ++i) {
-    const int hl = w + kWaves * i;
+    const int hl = hw0 + i;
     const bool sk = a.sink != nullptr && hl < nh && blockIdx.z == 0;
     m[i] = sk ? a.sink[h0 + hl] : -INFINITY;     // the sink: a key of score sink_h, no value
     l[i] = sk ? 1.f : 0.f;
+    sreg[i] = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[i][e] = 0.f;
   }
@@ -232,6 +240,7 @@ row_attn_kernel(const RowAttnArgs<T> a) {
   const bool vvec = (a.Dv % 8 == 0) && (a.vrow % 8 == 0);
   const int lpk = vvec ? a.Dv / 8 : 64, kpi = 64 / lpk;
   const int grp = lane / lpk, part = lane % lpk;
+  const int g_lo = h0 / hpg, g_hi = (h0 + nh - 1) / hpg;          // key/value heads of the block
   __syncthreads();
 
   int buf = 0;
@@ -245,34 +254,43 @@ row_attn_kernel(const RowAttnArgs<T> a) {
       const int key = lane & 15, kg = lane >> 4;
       const int jk = j0 + 16 * w + key;
       const long long rbk = jk <= pos ? (long long)tbl[jk / a.bs] * a.bs + jk % a.bs : 0;
-      const T* kp = a.kc + rbk * a.krow;
-      const T* qp = s_qb + key * (Dkp + kQPad);          // as B operand: the lane's head = lane & 15
-      f32x4v c = {0.f, 0.f, 0.f, 0.f};
       if (16 * w <= pos - j0) {                          // the wave's 16 keys hold a visible one
-        for (int d0 = 0; d0 < Dkp; d0 += 32) {
-          const int d = d0 + 8 * kg;
-          uint4 av = make_uint4(0u, 0u, 0u, 0u);
-          if (d < Dk) av = *reinterpret_cast<const uint4*>(kp + d);
-          const uint4 bv = *reinterpret_cast<const uint4*>(qp + d);
-          c = Mma16<T>::run(av, bv, c);
-        }
-      }
-      const int hl = lane & 15;                          // c[i] = S^T[key 4 kg + i][head hl]
-      if (hl < nh) {
-        const int h = h0 + hl;
+        for (int g = g_lo; g <= g_hi; ++g) {
+          const T* kp = a.kc + rbk * a.krow + (long long)g * Dk;
+          for (int nb = 0; nb < NB; ++nb) {
+            const int hl = 16 * nb + key;                // as B operand: the lane's head
+            if (16 * nb >= nh || (h0 + 16 * nb) / hpg > g || (h0 + min(nh, 16 * nb + 16) - 1) / hpg < g)
+              continue;                                  // none of these 16 heads uses g
+            const T* qp = s_qb + hl * (Dkp + kQPad);
+            f32x4v c = {0.f, 0.f, 0.f, 0.f};
+            for (int d0 = 0; d0 < Dkp; d0 += 32) {
+              const int d = d0 + 8 * kg;
+              uint4 av = make_uint4(0u, 0u, 0u, 0u);
+              if (d < Dk) av = *reinterpret_cast<const uint4*>(kp + d);
+              const uint4 bv = *reinterpret_cast<const uint4*>(qp + d);
+              c = Mma16<T>::run(av, bv, c);
+            }
+            if (hl < nh && (h0 + hl) / hpg == g) {       // c[i] = S^T[key 4 kg + i][head hl]
+              const int h = h0 + hl;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int kk = 16 * w + 4 * kg + i;
-          float sv = c[i] * qscale;
-          if (a.softcap > 0.f) sv = a.softcap * tanhf(sv / a.softcap);
-          if (a.r1 != nullptr) sv -= a.r1[h] * logf(1.f + a.r2[h] * (float)(pos - j0 - kk));
-          s_sc[(buf * a.HB + hl) * 64 + kk] = j0 + kk <= pos ? sv : 0.f;
+              for (int i = 0; i < 4; ++i) {
+                const int kk = 16 * w + 4 * kg + i;
+                float sv = c[i] * qscale;
+                if (a.softcap > 0.f) sv = a.softcap * tanhf(sv / a.softcap);
+                if (a.r1 != nullptr) sv -= a.r1[h] * logf(1.f + a.r2[h] * (float)(pos - j0 - kk));
+                s_sc[(buf * a.HB + hl) * 64 + kk] = j0 + kk <= pos ? sv : 0.f;
+              }
+            }
+          }
         }
+      } else {
+        for (int i = lane; i < 16 * nh; i += 64)         // no visible key: the scores are unused
+          s_sc[(buf * a.HB + i / 16) * 64 + 16 * w + i % 16] = 0.f;
       }
     } else {
 #pragma unroll
       for (int i = 0; i < HPW; ++i) {
-        const int hl = w + kWaves * i;
+        const int hl = hw0 + i;
         if (hl >= nh) break;
         const int h = h0 + hl;
         float dot = 0.f;
@@ -302,7 +320,7 @@ row_attn_kernel(const RowAttnArgs<T> a) {
     const int nk = min(64, pos - j0 + 1);
 #pragma unroll
     for (int i = 0; i < HPW; ++i) {
-      const int hl = w + kWaves * i;
+      const int hl = hw0 + i;
       if (hl >= nh) break;
       const int h = h0 + hl;
       float s = MMA ? s_sc[(buf * a.HB + hl) * 64 + lane] : sreg[i];
@@ -322,47 +340,60 @@ row_attn_kernel(const RowAttnArgs<T> a) {
     }
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    if (vvec && a.G == 1) {
-      // one key/value head: a value row is loaded once for all heads of the wave
-      if (grp < kpi) {
-        for (int jj = grp; jj < nk; jj += kpi) {
-          float vv[8];
-          load8<T>(a.vc + (long long)s_rb[buf * 64 + jj] * a.vrow + 8 * part, vv);
-#pragma unroll
-          for (int i = 0; i < HPW; ++i) {
-            const int hl = w + kWaves * i;
-            if (hl < nh) {
-              const float pj = s_p[hl * 64 + jj];
-#pragma unroll
-              for (int e = 0; e < 8; ++e) acc[i][e] += pj * vv[e];
-            }
-          }
-        }
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < HPW; ++i) {
-        const int hl = w + kWaves * i;
-        if (hl >= nh) break;
-        const long long voff = (long long)((h0 + hl) / hpg) * a.Dv;
+    if (hw0 < nh) {
+      // value pass: a value row is loaded once for all heads of the wave that share its
+      // key/value head, four rows in flight before their products
+      const int gw_lo = (h0 + hw0) / hpg, gw_hi = (h0 + min(nh, hw0 + HPW) - 1) / hpg;
+      for (int g = gw_lo; g <= gw_hi; ++g) {
+        const T* vbase = a.vc + (long long)g * a.Dv;
         if (vvec) {
           if (grp < kpi) {
-            for (int jj = grp; jj < nk; jj += kpi) {
-              const float pj = s_p[hl * 64 + jj];
-              float vv[8];
-              load8<T>(a.vc + (long long)s_rb[buf * 64 + jj] * a.vrow + voff + 8 * part, vv);
+            constexpr int U = 4;
+            for (int jj = grp; jj < nk; jj += kpi * U) {
+              Vec8<T> raw[U];
 #pragma unroll
-              for (int e = 0; e < 8; ++e) acc[i][e] += pj * vv[e];
+              for (int u = 0; u < U; ++u) {
+                const int k = min(jj + u * kpi, nk - 1);
+                raw[u] = *reinterpret_cast<const Vec8<T>*>(
+                    vbase + (long long)s_rb[buf * 64 + k] * a.vrow + 8 * part);
+              }
+#pragma unroll
+              for (int u = 0; u < U; ++u) {
+                const int k = jj + u * kpi;
+                if (k < nk) {
+                  float vv[8];
+#pragma unroll
+                  for (int e = 0; e < 8; ++e) vv[e] = to_f32(raw[u].v[e]);
+#pragma unroll
+                  for (int i = 0; i < HPW; ++i) {
+                    const int hl = hw0 + i;
+                    if (hl < nh && (h0 + hl) / hpg == g) {
+                      const float pj = s_p[hl * 64 + k];
+#pragma unroll
+                      for (int e = 0; e < 8; ++e) acc[i][e] += pj * vv[e];
+                    }
+                  }
+                }
+              }
             }
           }
         } else {
           for (int jj = 0; jj < nk; ++jj) {
-            const float pj = s_p[hl * 64 + jj];
-            const T* vp = a.vc + (long long)s_rb[buf * 64 + jj] * a.vrow + voff;
+            const T* vp = vbase + (long long)s_rb[buf * 64 + jj] * a.vrow;
+            float vv[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               const int d = lane + 64 * e;
-              if (d < a.Dv) acc[i][e] += pj * to_f32(vp[d]);
+              vv[e] = d < a.Dv ? to_f32(vp[d]) : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < HPW; ++i) {
+              const int hl = hw0 + i;
+              if (hl < nh && (h0 + hl) / hpg == g) {
+                const float pj = s_p[hl * 64 + jj];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[i][e] += pj * vv[e];
+              }
             }
           }
         }
@@ -374,7 +405,7 @@ row_attn_kernel(const RowAttnArgs<T> a) {
   float* so = s_o + w * kMaxDv;
 #pragma unroll
   for (int i = 0; i < HPW; ++i) {
-    const int hl = w + kWaves * i;
+    const int hl = hw0 + i;
     if (hl >= nh) break;
     const int h = h0 + hl;
     if (vvec) {
@@ -444,7 +475,7 @@ row_attn_combine_kernel(const float* __restrict__ ws_ml, const float* __restrict
 }
 
 inline size_t row_attn_lds(int HB, int Dk, bool mma = false, int esz = 2) {
-  const size_t q = mma ? ((size_t)16 * ((Dk + 31) / 32 * 32 + kQPad) * esz + 3) / 4 * 4
+  const size_t q = mma ? ((size_t)16 * ((HB + 15) / 16) * ((Dk + 31) / 32 * 32 + kQPad) * esz + 3) / 4 * 4
                        : sizeof(float) * (size_t)HB * Dk;
   return q + sizeof(float) * (3 * (size_t)HB * 64 + kWaves * kMaxDv) + sizeof(int) * 2 * 64;
 }
@@ -452,8 +483,11 @@ inline size_t row_attn_lds(int HB, int Dk, bool mma = false, int esz = 2) {
 template <typename T>
 bool row_attn_mma_ok(const RowAttnArgs<T>& a) {
   const int Dk = a.D1 + a.D2;
-  return Mma16<T>::ok && a.G == 1 && a.HB <= 16 && Dk % 8 == 0 && a.D1 % 8 == 0 &&
-         a.krow % 8 == 0 && ((uintptr_t)a.kc % 16 == 0);
+  const auto al = [](const void* p) { return (uintptr_t)p % 16 == 0; };
+  return Mma16<T>::ok && Dk % 8 == 0 && a.D1 % 8 == 0 && a.krow % 8 == 0 && al(a.kc) &&
+         al(a.q1) && a.q1r % 8 == 0 && a.q1h % 8 == 0 &&
+         (a.D2 == 0 || (al(a.q2) && a.q2r % 8 == 0 && a.q2h % 8 == 0)) &&
+         row_attn_lds(a.HB, Dk, true, sizeof(T)) <= 65536;
 }
 
 template <typename T>
@@ -468,7 +502,9 @@ hipError_t launch_row_attn(const RowAttnArgs<T>& a, int Tn, hipStream_t st) {
   if (mma) {
     if (hpw <= 1) LAUNCH(1, true);
     else if (hpw <= 2) LAUNCH(2, true);
-    else LAUNCH(4, true);
+    else if (hpw <= 4) LAUNCH(4, true);
+    else if (hpw <= 8) LAUNCH(8, true);
+    else return hipErrorInvalidValue;
   } else {
     if (hpw <= 1) LAUNCH(1, false);
     else if (hpw <= 2) LAUNCH(2, false);
