@@ -90,8 +90,8 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 latent_write_kernel(const T* __restrict__ z, long long ldz, const float* __restrict__ wn,
                     const float* __restrict__ inv_freq, const int* __restrict__ positions,
-                    const long long* __restrict__ slots, T* __restrict__ cache, int Tn, int R,
-                    int Dr, int dims, float eps) {
+                    const long long* __restrict__ slots, T* __restrict__ cache,
+                    T* __restrict__ vt, int bs, int Tn, int R, int Dr, int dims, float eps) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * kWaves + (threadIdx.x >> 6);
   if (t >= Tn) return;
@@ -106,7 +106,14 @@ latent_write_kernel(const T* __restrict__ z, long long ldz, const float* __restr
   }
   ss = wave_sum(ss);
   const float inv = 1.f / sqrtf(ss / (float)R + eps);
-  for (int c = lane; c < R; c += 64) dst[c] = from_f32<T>(to_f32(zr[c]) * inv * wn[c]);
+  // vt (optional): the normed latent once more, transposed per cache block [block][R][bs], for
+  // the matrix-core value product that contracts over the keys
+  T* dt = vt ? vt + (s / bs) * (long long)R * bs + s % bs : nullptr;
+  for (int c = lane; c < R; c += 64) {
+    const T v = from_f32<T>(to_f32(zr[c]) * inv * wn[c]);
+    dst[c] = v;
+    if (dt) dt[(long long)c * bs] = v;
+  }
   const float pos = (float)positions[t];
   for (int pr = lane; pr < dims / 2; pr += 64) {
     float sn, cs;
@@ -447,6 +454,215 @@ row_attn_kernel(const RowAttnArgs<T> a) {
   }
 }
 
+// ---- latent attention on the matrix cores -------------------------------------------------------
+// One key/value head whose value is the first Dv columns of the key row, 16-bit dtypes, Dv a
+// multiple of 64, cache blocks of a multiple of 8 tokens, and a second copy `vt` of the values
+// transposed per cache block, [block][Dv][bs].  A workgroup takes one row, up to 16 heads and 128
+// keys per step; wave w
+//   1. scores its own 32 keys against all heads: S^T = K Q^T (two 16-key tiles share the query
+//      operand from LDS), scales / caps / biases / masks them and takes their maxima per head;
+//   2. after the maxima of the four waves met in LDS: p = exp(s - max) for its keys, stored in LDS
+//      per head as a 16-bit head plus a 16-bit remainder (~16 mantissa bits of the fp32 weight);
+//   3. accumulates O^T = V^T P^T for ITS quarter of the value channels over all 128 keys: the A
+//      operand is 16 bytes of `vt` (8 consecutive keys of one channel), the B operand 16 bytes of
+//      the weights of one head; the accumulator's column is the head, so the running correction is
+//      lane-local and nothing is merged across waves at the end.
+// Scores, maxima, sums and the accumulator are fp32.
+template <typename T, int NT>   // NT: 16-channel tiles per wave, Dv = 64 NT
+__global__ void __launch_bounds__(64 * kWaves)
+latent_attn_kernel(const RowAttnArgs<T> a, const T* __restrict__ vt) {
+  extern __shared__ float smem[];
+  constexpr int kPRow = 128 + 8;                 // weights per head in LDS: 128 keys + padding
+  const int t = blockIdx.x, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int h0 = blockIdx.y * 16;
+  const int nh = min(16, a.H - h0);
+  const int Dk = a.D1 + a.D2;
+  const int Dkp = (Dk + 31) / 32 * 32;
+  const int pos = a.positions[t];
+  const int* tbl = a.tables + (long long)a.row_seg[t] * a.maxb;
+  const int hd = lane & 15, kg = lane >> 4;
+  T* s_qb = reinterpret_cast<T*>(smem);                               // [16][Dkp + pad]
+  T* s_ph = s_qb + 16 * (Dkp + kQPad);                                // [16][kPRow] head
+  T* s_pl = s_ph + 16 * kPRow;                                        // [16][kPRow] remainder
+  float* s_m = reinterpret_cast<float*>(s_pl + 16 * kPRow);           // [4][16]
+  float* s_l = s_m + kWaves * 16;                                     // [4][16]
+
+  const int cpr = Dkp / 8;
+  for (int c = threadIdx.x; c < 16 * cpr; c += 64 * kWaves) {
+    const int hl = c / cpr, d = (c % cpr) * 8;
+    const int h = h0 + hl;
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (hl < nh && d < Dk)
+      v = d < a.D1
+              ? *reinterpret_cast<const uint4*>(a.q1 + (long long)t * a.q1r + (long long)h * a.q1h + d)
+              : *reinterpret_cast<const uint4*>(a.q2 + (long long)t * a.q2r + (long long)h * a.q2h +
+                                                (d - a.D1));
+    *reinterpret_cast<uint4*>(s_qb + hl * (Dkp + kQPad) + d) = v;
+  }
+  float temp = 1.f;
+  if (a.tevery > 0 && a.tcoef != 0.f)
+    temp = 1.f + a.tcoef * logf((float)((pos + 1) / a.tevery) + 1.f);
+  const float qscale = a.scale * temp;
+  const bool head_on = hd < nh;
+  const int h = h0 + (head_on ? hd : 0);
+  const bool sk = a.sink != nullptr && blockIdx.z == 0;
+  float m_run = sk ? a.sink[h] : -INFINITY, l_run = sk ? 1.f : 0.f;
+  f32x4v O[NT];
+#pragma unroll
+  for (int n = 0; n < NT; ++n) O[n] = f32x4v{0.f, 0.f, 0.f, 0.f};
+  const T* qp = s_qb + hd * (Dkp + kQPad);
+  __syncthreads();
+
+  for (int j0 = 128 * blockIdx.z; j0 <= pos; j0 += 128 * a.nsplit) {
+    // 1. scores of the wave's 32 keys
+    const int jw = j0 + 32 * w;
+    float sc[2][4];
+    float mx = -INFINITY;
+    if (jw <= pos) {
+      f32x4v c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};
+      const int k0 = min(jw + hd, pos), k1 = min(jw + 16 + hd, pos);        // addressable keys
+      const T* kp0 = a.kc + ((long long)tbl[k0 / a.bs] * a.bs + k0 % a.bs) * a.krow;
+      const T* kp1 = a.kc + ((long long)tbl[k1 / a.bs] * a.bs + k1 % a.bs) * a.krow;
+      for (int d0 = 0; d0 < Dkp; d0 += 32) {
+        const int d = d0 + 8 * kg;
+        uint4 a0 = make_uint4(0u, 0u, 0u, 0u), a1 = a0;
+        if (d < Dk) {
+          a0 = *reinterpret_cast<const uint4*>(kp0 + d);
+          a1 = *reinterpret_cast<const uint4*>(kp1 + d);
+        }
+        const uint4 bv = *reinterpret_cast<const uint4*>(qp + d);
+        c0 = Mma16<T>::run(a0, bv, c0);
+        c1 = Mma16<T>::run(a1, bv, c1);
+      }
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int j = jw + 16 * sb + 4 * kg + i;         // c[i] = S^T[key 4 kg + i][head hd]
+          float sv = (sb ? c1[i] : c0[i]) * qscale;
+          if (a.softcap > 0.f) sv = a.softcap * tanhf(sv / a.softcap);
+          if (a.r1 != nullptr) sv -= a.r1[h] * logf(1.f + a.r2[h] * (float)(pos - j));
+          sv = j <= pos ? sv : -INFINITY;
+          sc[sb][i] = sv;
+          mx = fmaxf(mx, sv);
+        }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    } else {
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sc[sb][i] = -INFINITY;
+    }
+    if (kg == 0) s_m[w * 16 + hd] = mx;
+    __syncthreads();
+    // 2. the tile's maximum per head, the weights of the wave's keys into LDS
+    float mt = fmaxf(fmaxf(s_m[hd], s_m[16 + hd]), fmaxf(s_m[32 + hd], s_m[48 + hd]));
+    const float mn = fmaxf(m_run, mt);                     // finite: key j0 is visible
+    const float corr = expf(m_run - mn);
+    float ls = 0.f;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      float ph[4], pl[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = sc[sb][i] == -INFINITY ? 0.f : expf(sc[sb][i] - mn);
+        ls += pv;
+        ph[i] = to_f32(from_f32<T>(pv));
+        pl[i] = pv - ph[i];
+      }
+      const int col = 32 * w + 16 * sb + 4 * kg;
+      *reinterpret_cast<uint2*>(s_ph + hd * kPRow + col) = make_uint2(pk2<T>(ph[0], ph[1]), pk2<T>(ph[2], ph[3]));
+      *reinterpret_cast<uint2*>(s_pl + hd * kPRow + col) = make_uint2(pk2<T>(pl[0], pl[1]), pk2<T>(pl[2], pl[3]));
+    }
+    ls += __shfl_xor(ls, 16, 64);
+    ls += __shfl_xor(ls, 32, 64);
+    if (kg == 0) s_l[w * 16 + hd] = ls;
+#pragma unroll
+    for (int n = 0; n < NT; ++n) O[n] *= corr;
+    __syncthreads();
+    // 3. O^T += V^T P^T for the wave's channels over the tile's keys
+    l_run = l_run * corr + (s_l[hd] + s_l[16 + hd]) + (s_l[32 + hd] + s_l[48 + hd]);
+    m_run = mn;
+    for (int ks = 0; ks < 4; ++ks) {
+      const int jb = j0 + 32 * ks + 8 * kg;                // the lane's 8 keys
+      if (j0 + 32 * ks > pos) break;
+      const uint4 bh = *reinterpret_cast<const uint4*>(s_ph + hd * kPRow + 32 * ks + 8 * kg);
+      const uint4 bl = *reinterpret_cast<const uint4*>(s_pl + hd * kPRow + 32 * ks + 8 * kg);
+      const int ka = min(jb, pos);
+      const T* vp = vt + ((long long)tbl[ka / a.bs] * a.Dv) * a.bs + jb % a.bs;
+      // keys past the row's position carry weight 0 but may hold anything: blank them
+      const int nv = pos - jb + 1;                         // visible keys among the lane's 8
+      uint4 mk = make_uint4(~0u, ~0u, ~0u, ~0u);
+      if (nv < 8) {
+        const unsigned e = nv <= 0 ? 0u : (unsigned)nv;
+        const unsigned long long lo = e >= 4 ? ~0ull : (e == 0 ? 0ull : ((1ull << (16 * e)) - 1));
+        const unsigned long long hi = e <= 4 ? 0ull : ((1ull << (16 * (e - 4))) - 1);
+        mk = make_uint4((unsigned)lo, (unsigned)(lo >> 32), (unsigned)hi, (unsigned)(hi >> 32));
+      }
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        const int dv = (w * NT + n) * 16 + hd;             // as A operand: the lane's channel
+        uint4 av = *reinterpret_cast<const uint4*>(vp + (long long)dv * a.bs);
+        av.x &= mk.x; av.y &= mk.y; av.z &= mk.z; av.w &= mk.w;
+        O[n] = Mma16<T>::run(av, bh, O[n]);
+        O[n] = Mma16<T>::run(av, bl, O[n]);
+      }
+    }
+  }
+  // O[n][i] = O^T[channel (w NT + n) 16 + 4 kg + i][head hd]
+  if (head_on) {
+    if (a.nsplit == 1) {
+      const float inv = 1.f / l_run;
+      T* op = a.out + (long long)t * a.our + (long long)h * a.ouh;
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        const int dv = (w * NT + n) * 16 + 4 * kg;
+        *reinterpret_cast<uint2*>(op + dv) =
+            make_uint2(pk2<T>(O[n][0] * inv, O[n][1] * inv), pk2<T>(O[n][2] * inv, O[n][3] * inv));
+      }
+    } else {
+      const long long slot = ((long long)t * a.H + h) * a.nsplit + blockIdx.z;
+      if (w == 0 && kg == 0) {
+        a.ws_ml[2 * slot] = m_run;
+        a.ws_ml[2 * slot + 1] = l_run;
+      }
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        const int dv = (w * NT + n) * 16 + 4 * kg;
+        *reinterpret_cast<float4*>(a.ws_o + slot * a.Dv + dv) =
+            make_float4(O[n][0], O[n][1], O[n][2], O[n][3]);
+      }
+    }
+  }
+}
+
+inline size_t latent_attn_lds(int Dk, int esz) {
+  return (size_t)16 * ((Dk + 31) / 32 * 32 + kQPad) * esz + 2 * (size_t)16 * (128 + 8) * esz +
+         2 * kWaves * 16 * sizeof(float);
+}
+
+template <typename T>
+hipError_t launch_latent_attn(const RowAttnArgs<T>& a, const T* vt, int Tn, hipStream_t st) {
+  const size_t lds = latent_attn_lds(a.D1 + a.D2, sizeof(T));
+  const dim3 grid(Tn, (a.H + 15) / 16, a.nsplit);
+  switch (a.Dv / 64) {
+    case 1: latent_attn_kernel<T, 1><<<grid, 64 * kWaves, lds, st>>>(a, vt); break;
+    case 2: latent_attn_kernel<T, 2><<<grid, 64 * kWaves, lds, st>>>(a, vt); break;
+    case 3: latent_attn_kernel<T, 3><<<grid, 64 * kWaves, lds, st>>>(a, vt); break;
+    case 4: latent_attn_kernel<T, 4><<<grid, 64 * kWaves, lds, st>>>(a, vt); break;
+    case 6: latent_attn_kernel<T, 6><<<grid, 64 * kWaves, lds, st>>>(a, vt); break;
+    case 8: latent_attn_kernel<T, 8><<<grid, 64 * kWaves, lds, st>>>(a, vt); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+template <>
+hipError_t launch_latent_attn<float>(const RowAttnArgs<float>&, const float*, int, hipStream_t) {
+  return hipErrorInvalidValue;
+}
+
 // out[t, h] = sum_s acc_s exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s: the splits of a
 // row's keys merged; a split that saw no key has (m, l) = (-inf, 0) and drops out
 template <typename T>
@@ -542,11 +758,11 @@ hipError_t sm_rotate_heads(int dt, void* x, long long ldr, long long ldh, int he
 
 hipError_t sm_latent_write(int dt, const void* z, long long ldz, const float* wn,
                            const float* inv_freq, const int* positions, const long long* slots,
-                           void* cache, int T, int R, int Dr, int dims, float eps,
-                           hipStream_t st) {
+                           void* cache, void* vt, int bs, int T, int R, int Dr, int dims,
+                           float eps, hipStream_t st) {
   if (T == 0) return hipSuccess;
   if (dims % 2 || dims > Dr) return hipErrorInvalidValue;
-#define CALL(TT) latent_write_kernel<TT><<<(T + kWaves - 1) / kWaves, 256, 0, st>>>((const TT*)z, ldz, wn, inv_freq, positions, slots, (TT*)cache, T, R, Dr, dims, eps)
+#define CALL(TT) latent_write_kernel<TT><<<(T + kWaves - 1) / kWaves, 256, 0, st>>>((const TT*)z, ldz, wn, inv_freq, positions, slots, (TT*)cache, (TT*)vt, bs, T, R, Dr, dims, eps)
   SM_DISPATCH(dt, CALL)
 #undef CALL
   return hipGetLastError();
@@ -557,6 +773,52 @@ hipError_t sm_head_norm_write(int dt, void* qkv, long long ld, const float* wq, 
                               int G, int D, int Dv, float eps, hipStream_t st) {
   if (T == 0) return hipSuccess;
 #define CALL(TT) head_norm_write_kernel<TT><<<T, 256, 0, st>>>((TT*)qkv, ld, wq, wk, slots, (TT*)kcache, (TT*)vcache, H, G, D, Dv, eps)
+  SM_DISPATCH(dt, CALL)
+#undef CALL
+  return hipGetLastError();
+}
+
+// 1 when sm_latent_attn has a kernel for these sizes (dtype code dt, value size Dv = the latent,
+// key size Dk, cache block bs), else 0: the caller then takes sm_row_attn
+int sm_latent_attn_ok(int dt, int Dv, int Dk, int D1, int bs) {
+  if (dt != kBF16 && dt != kF16) return 0;
+  const int nt = Dv / 64;
+  return Dv % 64 == 0 && (nt == 1 || nt == 2 || nt == 3 || nt == 4 || nt == 6 || nt == 8) &&
+         Dk % 8 == 0 && D1 % 8 == 0 && Dv <= Dk && bs % 8 == 0 && latent_attn_lds(Dk, 2) <= 65536;
+}
+
+// Latent attention (one key/value head, values = the first Dv columns of a key row) with the
+// value product on the matrix cores; `vt` is the per-block transposed copy of the values that
+// sm_latent_write keeps.  Arguments as sm_row_attn (no head mixing); strides of q and out must be
+// multiples of 8 / 4 elements.
+hipError_t sm_latent_attn(int dt, const void* q1, long long q1r, long long q1h, int D1,
+                          const void* q2, long long q2r, long long q2h, int D2, const void* kc,
+                          long long krow, const void* vt, int Dv, void* out, long long our,
+                          long long ouh, const int* tables, int maxb, const int* row_seg,
+                          const int* positions, int T, int H, int bs, float scale, float softcap,
+                          float tcoef, int tevery, const float* r1, const float* r2,
+                          const float* sink, int nsplit, float* ws_ml, float* ws_o,
+                          hipStream_t st) {
+  if (T == 0) return hipSuccess;
+  const auto al = [](const void* p) { return (uintptr_t)p % 16 == 0; };
+  if (!sm_latent_attn_ok(dt, Dv, D1 + D2, D1, bs) || nsplit < 1 || nsplit > 64 ||
+      (nsplit > 1 && (!ws_ml || !ws_o)) || krow % 8 || !al(kc) || !al(vt) || !al(q1) || q1r % 8 ||
+      q1h % 8 || (D2 > 0 && (!q2 || !al(q2) || q2r % 8 || q2h % 8)) || our % 4 || ouh % 4 ||
+      (uintptr_t)out % 8)
+    return hipErrorInvalidValue;
+#define CALL(TT)                                                                              \
+  {                                                                                           \
+    RowAttnArgs<TT> a{(const TT*)q1, q1r, q1h, D1, (const TT*)q2, q2r, q2h, D2,               \
+                      (const TT*)kc, krow, (const TT*)kc, krow, Dv, (TT*)out, our, ouh,       \
+                      tables, maxb, row_seg, positions, H, 1, 16, bs, scale, softcap, tcoef,  \
+                      tevery, r1, r2, nullptr, sink, nsplit, ws_ml, ws_o};                    \
+    hipError_t e = launch_latent_attn<TT>(a, (const TT*)vt, T, st);                           \
+    if (e != hipSuccess) return e;                                                            \
+    if (nsplit > 1)                                                                           \
+      row_attn_combine_kernel<TT><<<dim3(T, H), 256, 0, st>>>(ws_ml, ws_o, (TT*)out, our,     \
+                                                              ouh, H, Dv, nsplit);            \
+    return hipGetLastError();                                                                 \
+  }
   SM_DISPATCH(dt, CALL)
 #undef CALL
   return hipGetLastError();

@@ -36,8 +36,9 @@ SIGNATURES = {
     "sm_group_rms": "iiplpppliiif",
     "sm_gate_rows": "iplplpiipi",
     "sm_rotate_heads": "iplliiippi",
-    "sm_latent_write": "iplpppppiiiif",
+    "sm_latent_write": "iplppppppiiiiif",
     "sm_head_norm_write": "iplpppppiiiiif",
+    "sm_latent_attn": "i" "plli" "plli" "pl" "pi" "pll" "pi" "pp" "iii" "fffi" "ppp" "ipp",
     "sm_row_attn": "i" "plli" "plli" "pl" "pli" "pll" "pi" "pp" "iiiii" "fffi" "pppp" "ipp",
 }
 
@@ -61,6 +62,8 @@ def _load():
         lib.sm_chunk_attn_tiles_ok.restype = ctypes.c_int
         lib.sm_row_attn_lds.argtypes = [ctypes.c_int, ctypes.c_int]
         lib.sm_row_attn_lds.restype = ctypes.c_int
+        lib.sm_latent_attn_ok.argtypes = [ctypes.c_int] * 5
+        lib.sm_latent_attn_ok.restype = ctypes.c_int
         _lib = lib
     except Exception as e:  # pragma: no cover - depends on build state
         _err = e
@@ -93,6 +96,11 @@ def tiles_ok(dt: int, D: int) -> bool:
 def row_attn_lds(HB: int, Dk: int) -> int:
     """LDS bytes the row-attention kernel needs for a block of HB heads with key size Dk."""
     return int(_load().sm_row_attn_lds(HB, Dk))
+
+
+def latent_attn_ok(dt: int, Dv: int, Dk: int, D1: int, bs: int) -> bool:
+    """Does the matrix-core latent attention have a kernel for these sizes?"""
+    return bool(_load().sm_latent_attn_ok(dt, Dv, Dk, D1, bs))
 
 
 def _arg(kind, v):

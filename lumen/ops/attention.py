@@ -588,7 +588,7 @@ def chunk_sink_attention(q: torch.Tensor, cache: torch.Tensor, seg, H: int, G: i
 # dot product and the softmax is a parameter: a position-dependent query temperature, a tanh soft
 # cap, a logarithmic distance bias per head, a mixing of the heads' scores, a per-head sink in
 # the softmax denominator.  Scores and weights are fp32.
-def latent_write_ref(z, w_norm, inv_freq, positions, slots, cache, R, dims, eps):
+def latent_write_ref(z, w_norm, inv_freq, positions, slots, cache, R, dims, eps, vt=None):
     zf = z.float()
     c = zf[:, :R]
     c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * w_norm.float()
@@ -599,25 +599,44 @@ def latent_write_ref(z, w_norm, inv_freq, positions, slots, cache, R, dims, eps)
     kr[:, 1:dims:2] = v * torch.cos(a) + u * torch.sin(a)
     ok = slots >= 0
     cache.view(-1, cache.shape[-1])[slots[ok]] = torch.cat([c, kr], 1)[ok].to(cache.dtype)
+    if vt is not None:
+        bs = vt.shape[2]
+        vt[slots[ok] // bs, :, slots[ok] % bs] = c[ok].to(vt.dtype)
+
+
+def transposed_values_ok(dtype, R: int, Dr: int, block_size: int, device) -> bool:
+    """Can latent attention over rows [R | Dr] run its value product on the matrix cores, i.e.
+    is a per-block transposed copy of the latents [blocks, R, block] worth keeping?"""
+    from ._seqmix import DT, latent_attn_ok
+
+    if torch.device(device).type != "cuda" or dtype not in (torch.bfloat16, torch.float16):
+        return False
+    return latent_attn_ok(DT[dtype], R, R + Dr, R, block_size)
 
 
 def latent_write(z: torch.Tensor, w_norm: torch.Tensor, inv_freq: torch.Tensor,
                  positions: torch.Tensor, slots: torch.Tensor, cache: torch.Tensor, R: int,
-                 dims: int, eps: float) -> None:
+                 dims: int, eps: float, vt: Optional[torch.Tensor] = None) -> None:
     """Rows of a latent-attention layer's down projection z [T, R + Dr] into the paged cache
     [blocks, block, R + Dr] at ``slots`` (int64; -1 skips): the first R columns RMS-normed with
-    ``w_norm``, the rest (the key part all heads share) rotated on its first ``dims`` columns."""
+    ``w_norm``, the rest (the key part all heads share) rotated on its first ``dims`` columns.
+    ``vt`` [blocks, R, block] (optional) takes the normed latents once more, transposed within
+    each cache block: the layout the matrix-core value product reads (keys contiguous)."""
     from ._seqmix import DT, call, use_seqmix
 
     Dr = z.shape[1] - R
     if cache.shape[-1] != R + Dr or dims > Dr or dims % 2:
         raise ValueError(f"latent row {R}+{Dr} (rotary {dims}) does not fit cache rows of "
                          f"{cache.shape[-1]}")
+    if vt is not None and (tuple(vt.shape) != (cache.shape[0], R, cache.shape[1])
+                           or vt.dtype != cache.dtype or not vt.is_contiguous()):
+        raise ValueError(f"transposed copy {tuple(vt.shape)} does not match cache "
+                         f"{tuple(cache.shape)} with latent size {R}")
     if not use_seqmix(z):
-        return latent_write_ref(z, w_norm, inv_freq, positions, slots, cache, R, dims, eps)
+        return latent_write_ref(z, w_norm, inv_freq, positions, slots, cache, R, dims, eps, vt)
     assert z.stride(1) == 1 and cache.is_contiguous() and cache.dtype == z.dtype
     call("sm_latent_write", DT[z.dtype], z, z.stride(0), w_norm, inv_freq, positions, slots, cache,
-         z.shape[0], R, Dr, dims, eps)
+         vt, cache.shape[1], z.shape[0], R, Dr, dims, eps)
 
 
 def head_norm_write_ref(qkv, wq, wk, slots, kcache, vcache, H, G, D, Dv, eps):
@@ -717,7 +736,7 @@ def _heads_per_block(H: int, Dk: int, need_all: bool) -> int:
 def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Tensor,
                   vcache: torch.Tensor, Dv: int, out: torch.Tensor, seg, H: int, G: int,
                   scale: float, softcap: float = 0.0, q_temp=None, r1=None, r2=None, talk=None,
-                  sink=None) -> torch.Tensor:
+                  sink=None, vt: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of every row of a step against paged caches.
 
     q1 [T, H, D1] and (optionally) q2 [T, H, D2] are views with arbitrary row / head strides;
@@ -729,8 +748,10 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).  ``softcap`` > 0: s <- cap *
     tanh(s / cap).  ``r1``, ``r2`` [H]: s <- s - r1 * ln(1 + r2 * distance).  ``talk`` [H, H]:
     the heads' scores are mixed, s_h <- sum_g talk[h, g] s_g.  ``sink`` [H]: exp(sink_h) joins
-    the softmax denominator."""
-    from ._seqmix import DT, call, use_seqmix
+    the softmax denominator.  ``vt`` [blocks, Dv, block]: a per-block transposed copy of the
+    values (``latent_write`` keeps one); with it, one key/value head, values that are a prefix of
+    the key rows and a 16-bit dtype, the whole kernel runs on the matrix cores."""
+    from ._seqmix import DT, call, latent_attn_ok, use_seqmix
 
     T, _, D1 = q1.shape
     D2 = q2.shape[2] if q2 is not None else 0
@@ -749,8 +770,28 @@ def row_attention(q1: torch.Tensor, q2: Optional[torch.Tensor], kcache: torch.Te
     assert krow >= G * Dk and vrow >= G * Dv
     for f in (r1, r2, talk, sink):
         assert f is None or (f.dtype == torch.float32 and f.is_contiguous())
-    HB = _heads_per_block(H, Dk, talk is not None)
     coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp is not None else (0.0, 0)
+    bs = kcache.shape[1]
+    al8 = lambda x: x.data_ptr() % 16 == 0 and x.stride(0) % 8 == 0 and x.stride(1) % 8 == 0  # noqa: E731
+    if (vt is not None and G == 1 and talk is None and vcache is kcache and D1 >= Dv
+            and q1.dtype in (torch.bfloat16, torch.float16) and latent_attn_ok(DT[q1.dtype], Dv, Dk, D1, bs)
+            and krow % 8 == 0 and al8(q1) and (q2 is None or al8(q2)) and out.data_ptr() % 8 == 0
+            and out.stride(0) % 4 == 0 and out.stride(1) % 4 == 0):
+        assert tuple(vt.shape) == (kcache.shape[0], Dv, bs) and vt.is_contiguous()
+        blocks = T * ((H + 15) // 16)
+        tiles = (seg.tables.shape[1] * bs + 127) // 128
+        nsplit = max(1, min(tiles, 32, 512 // max(blocks, 1)))
+        ws_ml = ws_o = None
+        if nsplit > 1:
+            ws_ml = torch.empty(T * H * nsplit * 2, dtype=torch.float32, device=q1.device)
+            ws_o = torch.empty(T * H * nsplit * Dv, dtype=torch.float32, device=q1.device)
+        call("sm_latent_attn", DT[q1.dtype], q1, q1.stride(0), q1.stride(1), D1,
+             q2, q2.stride(0) if q2 is not None else 0, q2.stride(1) if q2 is not None else 0, D2,
+             kcache, krow, vt, Dv, out, out.stride(0), out.stride(1),
+             seg.tables, seg.tables.shape[1], seg.row_seg, seg.positions, T, H, bs,
+             scale, float(softcap or 0.0), coef, every, r1, r2, sink, nsplit, ws_ml, ws_o)
+        return out
+    HB = _heads_per_block(H, Dk, talk is not None)
     # few rows (decoding): deal a row's 64-key tiles out to several workgroups so that ~2 per CU
     # run; the count depends on the step's size only, never on device data (graph capture)
     tiles = (seg.tables.shape[1] * kcache.shape[1] + 63) // 64

@@ -41,7 +41,7 @@ import torch.nn.functional as F
 from ..models.config import ModelConfig
 from ..models.gedatar import DELTA_DECAY, DELTA_KEY_EPS
 from ..ops.attention import (chunk_sink_attention, head_norm_write, latent_write, row_attention,
-                             write_key_cache)
+                             transposed_values_ok, write_key_cache)
 from ..ops.conv import dyt_canon
 from ..ops.embedding import gated_token_slice
 from ..ops.moe import gated_act, moe, route_topk
@@ -169,7 +169,7 @@ def key_bytes_per_token(cfg: ModelConfig, dtype_bytes: int = 2) -> int:
             if L["type"] == "attention":
                 n += m["kv_heads"] * (m["dim"] + m["vdim"])
             elif m.get("kv_from") is None:
-                n += m["kv_rank"] + m["rot_dim"]
+                n += 2 * m["kv_rank"] + m["rot_dim"]     # the latent twice: rows and transposed
         return max(1, n * dtype_bytes)
     return max(1, sum(L["mixer"]["kv_heads"] * L["mixer"]["dim"] for L in cfg.layer_specs
                       if L["type"] == "attention") * dtype_bytes)
@@ -340,8 +340,9 @@ class DalavikWeights:
 
 class DalavikState:
     """Paged caches of a Dalavik model: one row [latent | rotated key part] per token for every
-    latent-attention layer that projects its own (a borrowing layer reads the lender's), normed
-    keys and values for every grouped-query layer.  No per-sequence state: ``spare`` only names
+    latent-attention layer that projects its own (a borrowing layer reads the lender's) plus,
+    where the matrix-core value product can use it, the latents transposed within each block
+    [blocks, R, block]; normed keys and values for every grouped-query layer.  No per-sequence state: ``spare`` only names
     the slot number graph padding rows carry."""
 
     def __init__(self, w: DalavikWeights, slots: int, num_blocks: int, block_size: int, device):
@@ -349,6 +350,7 @@ class DalavikState:
         self.spare = slots
         kw = dict(dtype=w.dtype, device=device)
         self.lat: List[Optional[torch.Tensor]] = []
+        self.latT: List[Optional[torch.Tensor]] = []
         self.k: List[Optional[torch.Tensor]] = []
         self.v: List[Optional[torch.Tensor]] = []
         for i, L in enumerate(w.layers):
@@ -356,6 +358,9 @@ class DalavikState:
             own = L.kind == "latent_attention" and L.kv_layer == i
             self.lat.append(torch.zeros(num_blocks, block_size, m["kv_rank"] + m["rot_dim"], **kw)
                             if own else None)
+            self.latT.append(torch.zeros(num_blocks, m["kv_rank"], block_size, **kw)
+                             if own and transposed_values_ok(w.dtype, m["kv_rank"], m["rot_dim"],
+                                                             block_size, device) else None)
             att = L.kind == "attention"
             self.k.append(torch.zeros(num_blocks, block_size, m["kv_heads"], m["dim"], **kw)
                           if att else None)
@@ -382,7 +387,7 @@ def run_dalavik_layers(w: DalavikWeights, st: DalavikState, tokens: torch.Tensor
             z = F.linear(xb, L.w["down"])
             if L.kv_layer == i:
                 latent_write(z[:, Q:], L.w["dkv_norm"], L.w["inv_freq"], seg.positions,
-                             seg.cache_slots, st.lat[i], R, m["rot"]["dims"], eps)
+                             seg.cache_slots, st.lat[i], R, m["rot"]["dims"], eps, st.latT[i])
             cache = st.lat[L.kv_layer]
             q = F.linear(group_rms_norm(z[:, :Q], L.w["dq_norm"], 1, eps, dt), L.w["uq"])
             rotate_interleaved_(q, seg.positions, H, D + Dr, D, m["rot"]["dims"], L.w["inv_freq"])
@@ -390,7 +395,7 @@ def run_dalavik_layers(w: DalavikWeights, st: DalavikState, tokens: torch.Tensor
             qa = torch.bmm(q3[:, :, :D].transpose(0, 1), L.w["uk"])              # [H, T, R]
             ol = torch.empty(H, T, R, dtype=dt, device=x.device)
             row_attention(qa.transpose(0, 1), q3[:, :, D:], cache, cache, R, ol.transpose(0, 1),
-                          seg, H, 1, float(m["scale"]))
+                          seg, H, 1, float(m["scale"]), vt=st.latT[L.kv_layer])
             o = torch.empty(T, H, Dv, dtype=dt, device=x.device)
             torch.bmm(ol, L.w["uvT"], out=o.transpose(0, 1))
         else:

@@ -68,6 +68,12 @@ CONFIGS = {
         _att(1, 1, 16, 8, 0.4, _ff(40), softcap=3.0, q_temp=(0.7, 1)),
         _lat(1, 8, 4, 16, 40, 8, 0.25, 50.0, 4, _ff(24)),
         _att(8, 1, 8, 8, 0.35, None, q_temp=(0.05, 16))]),
+    # latents of 128 and cache blocks of 16: in 16 bits the value product of the latent layers
+    # runs on the matrix cores from the transposed copy; 18 heads make two head blocks
+    "wide": lambda: _cfg("wide", 200, 128, 2, 0, 1e-5, [
+        _lat(5, 32, 32, 24, 128, 48, 0.12, 10000.0, 32, _ff(96)),
+        _att(4, 2, 32, 32, 0.2, None, softcap=8.0),
+        _lat(18, 16, 32, 16, 128, 32, 0.15, 10000.0, 32, _ff(64), kv_from=0)]),
 }
 
 
@@ -393,16 +399,16 @@ def test_trace_run_command_line(tmp_path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name", ["tiny", "odd"])
+@pytest.mark.parametrize("name", ["tiny", "odd", "wide"])
 def test_bf16_close_to_oracle_and_cut_invariant(name):
     """bf16 serving: within rounding of the float64 oracle, and the same logits (to rounding)
     however the prompt is cut and whether rows decode through the hipGraph path or eagerly."""
     m = make(name, "cuda", dtype=torch.bfloat16, seed=9)
-    toks = tokens(m, 70, 50)
+    toks = tokens(m, 170 if name == "wide" else 70, 50)
     want = oracle(m).forward(toks)
     whole = replay_alone(m, "cuda", toks, [1000])
     cut = replay_alone(m, "cuda", toks, [7, 1, 2, 1, 1, 16])
-    eager = replay_alone(m, "cuda", toks, [30] + [1] * 50, graphs=False)
+    eager = replay_alone(m, "cuda", toks, [30] + [1] * 150, graphs=False)
     for got in (whole, cut, eager):
         check_rounding(got, want)
     check_rounding(cut, whole)

@@ -121,7 +121,9 @@ def test_latent_write(device, dtype, R, Dr, dims):
     pos = torch.tensor([0, 1, 2, 3, 40, 41, 500, 7, 8], dtype=torch.int32, device=device)
     slots = torch.tensor([5, 4, 63, -1, 0, 17, 33, 2, -1], device=device)
     cache = torch.full((4, 16, R + Dr), 9.0, dtype=dtype, device=device)
-    latent_write(z, wn, interleaved_inv_freq(dims, 300.0, device), pos, slots, cache, R, dims, 1e-5)
+    vt = torch.full((4, R, 16), 9.0, dtype=dtype, device=device)
+    latent_write(z, wn, interleaved_inv_freq(dims, 300.0, device), pos, slots, cache, R, dims, 1e-5,
+                 vt)
     zf = z.cpu().to(F64)
     c = ref.rms_unit(zf[:, :R], 1e-5) * wn.cpu().to(F64)
     kr = ref.rotate_pairs(zf[:, R:], pos.cpu(), dims, 300.0)
@@ -133,6 +135,8 @@ def test_latent_write(device, dtype, R, Dr, dims):
             close(rows[s], torch.cat([c[t], kr[t]]), dtype)
     for s in set(range(64)) - used:                      # skipped rows and the rest stay untouched
         assert bool((rows[s] == 9.0).all())
+    # the transposed copy holds the same latents, [block][R][token in block]
+    assert torch.equal(vt.transpose(1, 2).reshape(64, R).cpu(), rows[:, :R])
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
@@ -253,10 +257,14 @@ def test_row_attention_grouped_with_everything(device, dtype, H, G, D, Dv, bs):
 
 @pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("H,D1,D2,R,bs", [(3, 32, 8, 32, 8), (7, 22, 6, 22, 16), (16, 64, 16, 64, 16),
-                                          (5, 128, 32, 128, 16)])
-def test_row_attention_latent_two_part_query(device, dtype, H, D1, D2, R, bs):
+                                          (5, 128, 32, 128, 16), (20, 192, 24, 192, 8),
+                                          (9, 512, 64, 512, 16)])
+@pytest.mark.parametrize("transposed", [False, True])
+def test_row_attention_latent_two_part_query(device, dtype, H, D1, D2, R, bs, transposed):
     """One shared cache row per token, the value its first R columns, the query in two parts
-    with strides of their own (head-major and token-major), the output written head-major."""
+    with strides of their own (head-major and token-major), the output written head-major; with
+    and without the per-block transposed copy of the values that switches the matrix-core value
+    product on where it has a kernel (16-bit, R a multiple of 64)."""
     assert D1 == R
     rows = [rnd(n, R + D2, seed=50 + i, dtype=dtype) for i, n in enumerate(LENS)]
     cache, tb = paged(rows, bs, 40, R + D2, dtype, device, 2)
@@ -265,15 +273,19 @@ def test_row_attention_latent_two_part_query(device, dtype, H, D1, D2, R, bs):
     qa = rnd(H, T, D1, seed=60, dtype=dtype, device=device)                  # [H, T, D1]
     qb = rnd(T, H, 11 + D2, seed=61, dtype=dtype, device=device)[:, :, 11:]  # [T, H, D2], strided
     out = torch.zeros(H, T, R, dtype=dtype, device=device)
-    row_attention(qa.transpose(0, 1), qb, cache, cache, R, out.transpose(0, 1), seg, H, 1, 0.2)
+    vt = cache[:, :, :R].transpose(1, 2).contiguous() if transposed else None
+    sink = rnd(H, seed=62, device=device) if transposed else None
+    row_attention(qa.transpose(0, 1), qb, cache, cache, R, out.transpose(0, 1), seg, H, 1, 0.2,
+                  sink=sink, vt=vt)
     q = torch.cat([qa.transpose(0, 1), qb], -1).cpu()
     hg = torch.zeros(H, dtype=torch.long)
     at = 0
     for s, p0, n in SPANS:
         kv = rows[s][:p0 + n]
         want = dense_attention(q[at:at + n], kv.view(-1, 1, R + D2), kv[:, :R].reshape(-1, 1, R),
-                               torch.arange(p0, p0 + n), hg, 0.2)
-        close(out.transpose(0, 1)[at:at + n], want, dtype, scale=1.0)
+                               torch.arange(p0, p0 + n), hg, 0.2,
+                               sink=sink.cpu() if sink is not None else None)
+        close(out.transpose(0, 1)[at:at + n], want, dtype, scale=max(1.0, (D1 + D2) ** 0.5 / 8))
         at += n
 
 
