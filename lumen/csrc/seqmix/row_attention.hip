@@ -125,7 +125,7 @@ latent_write_kernel(const T* __restrict__ z, long long ldz, const float* __restr
   for (int c = dims + lane; c < Dr; c += 64) dst[R + c] = zr[R + c];
 }
 
-template <typename T>
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(256)
 head_norm_write_kernel(T* __restrict__ qkv, long long ld, const float* __restrict__ wq,
                        const float* __restrict__ wk, const long long* __restrict__ slots,
@@ -134,30 +134,64 @@ head_norm_write_kernel(T* __restrict__ qkv, long long ld, const float* __restric
   const int t = blockIdx.x, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const long long s = slots[t];
   T* row = qkv + (long long)t * ld;
+  constexpr int V = VEC ? 4 : 1;                 // elements per lane and step
   for (int item = w; item < H + 2 * G; item += kWaves) {
     if (item < H + G) {
       const bool is_q = item < H;
       T* src = row + (long long)item * D;           // q heads, then k heads, are consecutive
+      T* dst = is_q ? src : (s >= 0 ? kcache + (s * G + (item - H)) * D : nullptr);
+      const float* wt = is_q ? wq : wk;
       float ss = 0.f;
-      for (int c = lane; c < D; c += 64) {
-        const float v = to_f32(src[c]);
-        ss += v * v;
+      for (int c = V * lane; c < D; c += 64 * V) {
+        if (VEC) {
+          float v[4];
+          load4<T>(src + c, v);
+          ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+        } else {
+          const float v = to_f32(src[c]);
+          ss += v * v;
+        }
       }
       ss = wave_sum(ss);
       const float inv = 1.f / sqrtf(ss / (float)D + eps);
-      if (is_q) {
-        for (int c = lane; c < D; c += 64) src[c] = from_f32<T>(to_f32(src[c]) * inv * wq[c]);
-      } else if (s >= 0) {
-        T* dst = kcache + (s * G + (item - H)) * D;
-        for (int c = lane; c < D; c += 64) dst[c] = from_f32<T>(to_f32(src[c]) * inv * wk[c]);
+      if (dst) {
+        for (int c = V * lane; c < D; c += 64 * V) {
+          if (VEC) {
+            float v[4], ww[4];
+            load4<T>(src + c, v);
+            load4<float>(wt + c, ww);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = v[e] * inv * ww[e];
+            store4<T>(dst + c, v);
+          } else {
+            dst[c] = from_f32<T>(to_f32(src[c]) * inv * wt[c]);
+          }
+        }
       }
     } else if (s >= 0) {
       const int g = item - H - G;
       const T* src = row + (long long)(H + G) * D + (long long)g * Dv;
       T* dst = vcache + (s * G + g) * Dv;
-      for (int c = lane; c < Dv; c += 64) dst[c] = src[c];
+      for (int c = V * lane; c < Dv; c += 64 * V) {
+        if (VEC) {
+          float v[4];
+          load4<T>(src + c, v);
+          store4<T>(dst + c, v);
+        } else {
+          dst[c] = src[c];
+        }
+      }
     }
   }
+}
+
+// Workgroups are handed to the 8 XCDs round-robin in launch order, and every XCD has an L2 of its
+// own.  Rows that follow each other in a step belong to one sequence and read the same cache
+// blocks, so XCD x takes the x-th CONTIGUOUS eighth of the rows instead of every eighth row:
+// workgroup b -> row start(b % 8) + b / 8 (a bijection for any row count).
+__device__ __forceinline__ int xcd_row(int b, int n) {
+  const int q = n / 8, r = n % 8, x = b % 8;
+  return x * q + min(x, r) + b / 8;
 }
 
 template <typename T>
@@ -185,7 +219,7 @@ template <typename T, int HPW, bool MMA>
 __global__ void __launch_bounds__(64 * kWaves)
 row_attn_kernel(const RowAttnArgs<T> a) {
   extern __shared__ float smem[];
-  const int t = blockIdx.x, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int t = xcd_row(blockIdx.x, gridDim.x), lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int h0 = blockIdx.y * a.HB;
   const int nh = min(a.HB, a.H - h0);
   const int Dk = a.D1 + a.D2;
@@ -473,7 +507,7 @@ __global__ void __launch_bounds__(64 * kWaves)
 latent_attn_kernel(const RowAttnArgs<T> a, const T* __restrict__ vt) {
   extern __shared__ float smem[];
   constexpr int kPRow = 128 + 8;                 // weights per head in LDS: 128 keys + padding
-  const int t = blockIdx.x, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int t = xcd_row(blockIdx.x, gridDim.x), lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int h0 = blockIdx.y * 16;
   const int nh = min(16, a.H - h0);
   const int Dk = a.D1 + a.D2;
@@ -772,7 +806,14 @@ hipError_t sm_head_norm_write(int dt, void* qkv, long long ld, const float* wq, 
                               const long long* slots, void* kcache, void* vcache, int T, int H,
                               int G, int D, int Dv, float eps, hipStream_t st) {
   if (T == 0) return hipSuccess;
-#define CALL(TT) head_norm_write_kernel<TT><<<T, 256, 0, st>>>((TT*)qkv, ld, wq, wk, slots, (TT*)kcache, (TT*)vcache, H, G, D, Dv, eps)
+  const bool vec = D % 4 == 0 && Dv % 4 == 0 && ld % 4 == 0 && (uintptr_t)qkv % 16 == 0 &&
+                   (uintptr_t)kcache % 16 == 0 && (uintptr_t)vcache % 16 == 0 &&
+                   (uintptr_t)wq % 16 == 0 && (uintptr_t)wk % 16 == 0;
+#define CALL(TT)                                                                               \
+  if (vec) head_norm_write_kernel<TT, true><<<T, 256, 0, st>>>((TT*)qkv, ld, wq, wk, slots,   \
+                                                (TT*)kcache, (TT*)vcache, H, G, D, Dv, eps);   \
+  else head_norm_write_kernel<TT, false><<<T, 256, 0, st>>>((TT*)qkv, ld, wq, wk, slots,      \
+                                                 (TT*)kcache, (TT*)vcache, H, G, D, Dv, eps)
   SM_DISPATCH(dt, CALL)
 #undef CALL
   return hipGetLastError();
