@@ -256,7 +256,7 @@ def test_row_attention_grouped_with_everything(device, dtype, H, G, D, Dv, bs):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
-@pytest.mark.parametrize("H,D1,D2,R,bs", [(3, 32, 8, 32, 8), (7, 22, 6, 22, 16), (16, 64, 16, 64, 16),
+@pytest.mark.parametrize("H,D1,D2,R,bs", [(3, 32, 8, 32, 8), (7, 22, 6, 22, 16), (12, 64, 24, 64, 16),
                                           (5, 128, 32, 128, 16), (20, 192, 24, 192, 8),
                                           (9, 512, 64, 512, 16)])
 @pytest.mark.parametrize("transposed", [False, True])
