@@ -313,6 +313,63 @@ def test_preemption_recomputes_caches(device):
             assert float(row.max() - row[tok]) <= 1e-3 * max(float(row.std()), 1.0)
 
 
+def _random_config(seed):
+    """A random stack: 2 - 5 layers of either mixer in any order, borrowers of earlier caches,
+    sizes that are and are not multiples of the vector and matrix-core widths."""
+    import random
+
+    rng = random.Random(seed)
+    W = rng.choice([64, 96, 160, 192])
+    groups = rng.choice([g for g in (1, 2, 3, 4, 5, 8) if W % g == 0])
+    layers, lenders = [], []
+    for i in range(rng.randint(2, 5)):
+        mlp = _ff(rng.choice([32, 48, 100])) if rng.random() < 0.8 else None
+        if rng.random() < 0.6:
+            if lenders and rng.random() < 0.4:
+                src = rng.choice(lenders)
+                o = layers[src]["mixer"]
+                R, Dr, rot = o["kv_rank"], o["rot_dim"], o["rot"]
+            else:
+                src = None
+                R, Dr = rng.choice([16, 24, 64, 72, 128]), rng.choice([4, 6, 8, 16, 32])
+                rot = {"base": rng.choice([100.0, 10000.0, 500000.0]),
+                       "dims": Dr if rng.random() < 0.7 else max(2, Dr // 4 * 2)}
+            layers.append(_lat(rng.choice([1, 2, 3, 5, 8, 16, 17]), rng.choice([8, 12, 16, 40, 64]), Dr,
+                               rng.choice([8, 16, 20, 32]), R, rng.choice([16, 24, 48]),
+                               rng.uniform(0.05, 0.3), rot["base"], rot["dims"], mlp, src))
+            if src is None:
+                lenders.append(i)
+        else:
+            H = rng.choice([1, 2, 3, 4, 6, 8, 12, 32])
+            G = rng.choice([g for g in (1, 2, 3, 4, H) if H % g == 0])
+            layers.append(_att(H, G, rng.choice([8, 16, 20, 32, 64]), rng.choice([8, 12, 16, 48]),
+                               rng.uniform(0.05, 0.3), mlp, softcap=rng.choice([None, 5.0, 30.0]),
+                               q_temp=rng.choice([None, (0.3, 1), (0.2, 16), (0.1, 64)])))
+    return _cfg(f"random{seed}", rng.randint(50, 400), W, groups, rng.choice([0, 4, 12, 16]),
+                rng.choice([1e-6, 1e-5]), layers)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_random_configurations(device, seed):
+    """Whole, in ragged portions, and decoded across a 128-key border: the oracle's logits (fp32)
+    and, on the GPU in 16 bits, the same logits however the prompt was cut."""
+    cfg = _random_config(seed)
+    m = DalavikForCausalLM(cfg, dtype=torch.float32, device=device)
+    m.init_weights(seed=seed)
+    toks = tokens(m, 150, seed)
+    want = oracle(m).forward(toks)
+    for pieces in ([1000], [37, 2, 1, 50, 1, 1, 1, 3], [120] + [1] * 30):
+        check(replay_alone(m, device, toks, pieces), want, rtol=5e-4)
+    if device == "cuda":
+        m16 = DalavikForCausalLM(cfg, dtype=torch.bfloat16, device=device)
+        m16.init_weights(seed=seed)
+        whole = replay_alone(m16, device, toks, [1000])
+        check_rounding(replay_alone(m16, device, toks, [37, 2, 1, 50, 1, 1, 1, 3]), whole, rms=1e-2,
+                       worst=0.25)
+        check_rounding(replay_alone(m16, device, toks, [120] + [1] * 30), whole, rms=1e-2, worst=0.25)
+
+
 def test_configuration_is_validated():
     bad = CONFIGS["odd"]()
     bad.layer_specs[2]["mixer"]["kv_from"] = 3            # a later layer cannot lend its cache
